@@ -16,8 +16,146 @@ class PlainOps:
     def __init__(self, work=torch.float32):
         self.work = work
 
-    def embedding(self, ids, table, out):
-        out.copy_(table[ids.long()].to(torch.float32))
+    def embedding(self, ids, table, out, scale=1.0):
+        out.copy_((table[ids.long()].to(self.work) * scale).to(torch.float32))
+        return out
+
+    def add_pair_rmsnorm(self, residual, first, second, weight, eps, out, rows=None, store_residual=True):
+        pick = (lambda t: t) if rows is None else (lambda t: t[rows.long()])
+        x = pick(residual).to(self.work) + (pick(first).to(self.work) + pick(second).to(self.work))
+        if store_residual:
+            assert rows is None
+            residual.copy_(x.to(torch.float32))
+            x = residual.to(self.work)
+        if weight is not None:
+            x = x / torch.sqrt((x * x).mean(dim=-1, keepdim=True) + eps) * weight.to(self.work)
+        out.copy_(x.to(out.dtype))
+        return out
+
+    # ------------------------------------------------------------ attention over a cached latent
+    def _turn(self, x, positions, rates):
+        """Coordinate j < n/2 of the last axis with coordinate j + n/2, by position * rates[j] (float32 angles)."""
+        half = x.shape[-1] // 2
+        angles = positions.to(torch.float32)[:, None] * rates.to(torch.float32)[None, :]
+        cos, sin = angles.cos().to(self.work), angles.sin().to(self.work)
+        while cos.dim() < x.dim():
+            cos, sin = cos.unsqueeze(1), sin.unsqueeze(1)
+        a, b = x[..., :half], x[..., half:]
+        return torch.cat([a * cos - b * sin, b * cos + a * sin], dim=-1)
+
+    def latent_store(self, rows, q_offset, q_rank, q_norm, kv_offset, kv_rank, kv_norm, rot_dim, rates, eps, positions,
+                     slots, k_pages, v_pages, latent_q):
+        x = rows.to(self.work)
+        latent_q.copy_((self._unit(x[:, q_offset:q_offset + q_rank], eps) * q_norm.to(self.work)).to(latent_q.dtype))
+        kept = self._unit(x[:, kv_offset:kv_offset + kv_rank], eps) * kv_norm.to(self.work)
+        if rot_dim:
+            tail = x[:, kv_offset + kv_rank:kv_offset + kv_rank + rot_dim]
+            kept = torch.cat([kept, self._turn(tail, positions, rates)], dim=1)
+        if slots is None:
+            return
+        page_size = k_pages.shape[2]
+        kept = kept.to(k_pages.dtype)
+        for t in range(rows.shape[0]):
+            slot = int(slots[t])
+            if slot < 0:
+                continue
+            page, off = divmod(slot, page_size)
+            k_pages[page, 0, off, :] = kept[t]
+            v_pages[page, 0, :, off] = kept[t]
+
+    def head_linear(self, x, x_offset, x_head_stride, weight, out, out_offset, out_head_stride):
+        heads, n, k = weight.shape
+        for h in range(heads):
+            a = x[:, h * x_head_stride + x_offset:h * x_head_stride + x_offset + k].to(self.work)
+            at = h * out_head_stride + out_offset
+            out[:, at:at + n] = (a @ weight[h].to(self.work).t()).to(out.dtype)
+        return out
+
+    def rotate_tails(self, q, heads, head_width, tail_offset, dims, rates, positions, out, out_head_stride, out_offset):
+        x = q.to(self.work).reshape(q.shape[0], heads, head_width)[:, :, tail_offset:tail_offset + dims]
+        turned = self._turn(x, positions, rates).to(out.dtype)
+        for h in range(heads):
+            at = h * out_head_stride + out_offset
+            out[:, at:at + dims] = turned[:, h]
+        return out
+
+    # ------------------------------------------------------------ delta rule with a decay per key channel
+    def short_conv_silu(self, rows, offsets, widths, taps, state, state_offset, cu_q, first_position, state_slots,
+                        entry_of_token, out):
+        w = self.work
+        n_taps, channels = taps.shape[1], sum(widths)
+        x = torch.cat([rows[:, o:o + n] for o, n in zip(offsets, widths)], dim=1).to(w)
+        for e in range(cu_q.numel() - 1):
+            lo, hi = int(cu_q[e]), int(cu_q[e + 1])
+            if hi <= lo:
+                continue
+            slot = int(state_slots[e])
+            tail = state[slot, state_offset:state_offset + (n_taps - 1) * channels].to(w).reshape(n_taps - 1, channels)
+            if int(first_position[e]) == 0:
+                tail = torch.zeros_like(tail)
+            seen = torch.cat([tail, x[lo:hi]], dim=0)
+            y = torch.zeros((hi - lo, channels), dtype=w)
+            for j in range(n_taps):
+                y = y + seen[j:j + hi - lo] * taps[:, j].to(w)
+            out[lo:hi] = (y * torch.sigmoid(y)).to(out.dtype)
+            state[slot, state_offset:state_offset + (n_taps - 1) * channels] = seen[seen.shape[0] - (n_taps - 1):].reshape(-1).to(state.dtype)
+        return out
+
+    def delta_scan(self, fresh, decay, neg_rate, rows, beta_offset, state, cu_q, first_position, state_slots, out,
+                   heads, groups, d, dv, unit_eps):
+        w = self.work
+        share = heads // groups
+        for e in range(cu_q.numel() - 1):
+            lo, hi = int(cu_q[e]), int(cu_q[e + 1])
+            if hi <= lo:
+                continue
+            slot = int(state_slots[e])
+            S = state[slot, :heads * d * dv].to(w).reshape(heads, d, dv).clone()
+            if int(first_position[e]) == 0:
+                S = torch.zeros_like(S)
+            for t in range(lo, hi):
+                q = fresh[t, :groups * d].to(w).reshape(groups, d)
+                k = fresh[t, groups * d:2 * groups * d].to(w).reshape(groups, d)
+                v = fresh[t, 2 * groups * d:].to(w).reshape(heads, dv)
+                q = (q / torch.sqrt((q * q).sum(-1, keepdim=True) + unit_eps) * d ** -0.5).repeat_interleave(share, dim=0)
+                k = (k / torch.sqrt((k * k).sum(-1, keepdim=True) + unit_eps)).repeat_interleave(share, dim=0)
+                beta = torch.sigmoid(rows[t, beta_offset:beta_offset + heads].to(w))
+                g = torch.exp(neg_rate.to(w)[:, None] * torch.nn.functional.softplus(decay[t].to(w).reshape(heads, d)))
+                S = g[:, :, None] * S
+                u = beta[:, None] * (v - torch.einsum("hdv,hd->hv", S, k))
+                S = S + k[:, :, None] * u[:, None, :]
+                out[t] = torch.einsum("hdv,hd->hv", S, q).reshape(-1).to(out.dtype)
+            state[slot, :heads * d * dv] = S.reshape(-1).to(state.dtype)
+        return out
+
+    # ------------------------------------------------------------ sigmoid router with groups, ungated experts
+    def route_sigmoid(self, logits, correction, n_groups, keep_groups, chosen, weights):
+        top = chosen.shape[1]
+        s = torch.sigmoid(logits.to(torch.float32))
+        choice = s + correction.to(torch.float32)
+        if n_groups:
+            per = logits.shape[1] // n_groups
+            grouped = choice.reshape(-1, n_groups, per)
+            worth = torch.topk(grouped, min(2, per), dim=-1).values.sum(-1)
+            best = torch.topk(worth, keep_groups, dim=-1).indices
+            allowed = torch.zeros_like(worth, dtype=torch.bool).scatter_(1, best, True)
+            choice = grouped.masked_fill(~allowed[:, :, None], float("-inf")).reshape(choice.shape)
+        ids = torch.topk(choice, top, dim=-1).indices
+        picked = torch.gather(s, 1, ids)
+        chosen.copy_(ids.to(torch.int32))
+        weights.copy_(picked / (picked.sum(-1, keepdim=True) + 1e-20))
+
+    def expert_act(self, up, chosen, weights, n_experts, inner, out):
+        n_tokens = up.shape[0]
+        x = torch.relu(up.to(self.work)).pow(2).reshape(n_tokens, n_experts, inner)
+        factor = torch.zeros((n_tokens, n_experts), dtype=self.work)
+        factor.scatter_(1, chosen.long(), weights.to(self.work))
+        out.zero_()
+        out[:, :n_experts * inner] = (factor[:, :, None] * x).reshape(n_tokens, -1).to(out.dtype)
+        return out
+
+    def relu2(self, x, out):
+        out.copy_(torch.relu(x.to(self.work)).pow(2).to(out.dtype))
         return out
 
     def add_rmsnorm(self, residual, delta, weight, eps, out, rows=None, store_residual=True):

@@ -4,7 +4,8 @@ from .registry import (Architecture, architecture_name, get_architecture, load_c
 from .qwen2 import Qwen2Config
 from .napadra import NapadraConfig
 from .dolidra import DolidraConfig
+from .bokulorn import BokulornConfig
 
 __all__ = ["ConfigError", "ModelConfig", "read_config_json", "Architecture", "architecture_name",
            "get_architecture", "load_config", "register_architecture", "registered_architectures",
-           "Qwen2Config", "NapadraConfig", "DolidraConfig"]
+           "Qwen2Config", "NapadraConfig", "DolidraConfig", "BokulornConfig"]

@@ -1,23 +1,23 @@
 // Embedding gather, residual-add + RMSNorm, gated activation.
 #include "common.h"
 
-// out[t, :] = table[ids[t], :] widened to float (the residual stream is float).
+// out[t, :] = table[ids[t], :] widened to float (the residual stream is float), times `scale`.
 template <typename T>
 __global__ void embedding_kernel(const int* __restrict__ ids, const T* __restrict__ table,
-                                 float* __restrict__ out, int hidden, int vocab) {
+                                 float* __restrict__ out, int hidden, int vocab, float scale) {
   const int t = blockIdx.x;
   int id = ids[t];
   if (id < 0 || id >= vocab) id = 0;  // the host rejects such ids before the launch
   const T* row = table + (size_t)id * hidden;
   float* dst = out + (size_t)t * hidden;
-  for (int h = threadIdx.x; h < hidden; h += blockDim.x) dst[h] = ld(row + h);
+  for (int h = threadIdx.x; h < hidden; h += blockDim.x) dst[h] = ld(row + h) * scale;
 }
 
 // The same for bfloat16 tables whose rows are a multiple of eight long: sixteen bytes a thread.
 __global__ void __launch_bounds__(256)
 embedding_vec_kernel(const int* __restrict__ ids, const bf16_t* __restrict__ table, float* __restrict__ out,
-                     int hidden, int vocab) {
-  HELD(ids, table, out, hidden, vocab);
+                     int hidden, int vocab, float scale) {
+  HELD(ids, table, out, hidden, vocab, scale);
   const int t = blockIdx.x;
   int id = scalar_int(ids + t);
   if (id < 0 || id >= vocab) id = 0;  // the host rejects such ids before the launch
@@ -29,8 +29,8 @@ embedding_vec_kernel(const int* __restrict__ ids, const bf16_t* __restrict__ tab
     float v[8];
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      v[2 * i] = __uint_as_float(w[i] << 16);
-      v[2 * i + 1] = __uint_as_float(w[i] & 0xffff0000u);
+      v[2 * i] = __uint_as_float(w[i] << 16) * scale;
+      v[2 * i + 1] = __uint_as_float(w[i] & 0xffff0000u) * scale;
     }
     *reinterpret_cast<float4*>(dst + h8 * 8) = make_float4(v[0], v[1], v[2], v[3]);
     *reinterpret_cast<float4*>(dst + h8 * 8 + 4) = make_float4(v[4], v[5], v[6], v[7]);
@@ -267,14 +267,66 @@ __global__ void capped_gate_vec_kernel(const bf16_t* __restrict__ in, bf16_t* __
 }
 
 extern "C" int ta_embedding(const void* ids, const void* table, void* out, int n_tokens, int hidden,
-                            int vocab, int dtype, hipStream_t stream) {
+                            int vocab, int dtype, float scale, hipStream_t stream) {
   if (n_tokens <= 0) return 0;
   if (dtype == DT_F32)
-    embedding_kernel<float><<<n_tokens, 256, 0, stream>>>((const int*)ids, (const float*)table, (float*)out, hidden, vocab);
+    embedding_kernel<float><<<n_tokens, 256, 0, stream>>>((const int*)ids, (const float*)table, (float*)out, hidden, vocab, scale);
   else if (hidden % 8 == 0 && (((uintptr_t)table | (uintptr_t)out) & 15) == 0)
-    embedding_vec_kernel<<<n_tokens, 256, 0, stream>>>((const int*)ids, (const bf16_t*)table, (float*)out, hidden, vocab);
+    embedding_vec_kernel<<<n_tokens, 256, 0, stream>>>((const int*)ids, (const bf16_t*)table, (float*)out, hidden, vocab, scale);
   else
-    embedding_kernel<bf16_t><<<n_tokens, 256, 0, stream>>>((const int*)ids, (const bf16_t*)table, (float*)out, hidden, vocab);
+    embedding_kernel<bf16_t><<<n_tokens, 256, 0, stream>>>((const int*)ids, (const bf16_t*)table, (float*)out, hidden, vocab, scale);
+  return LAUNCH_STATUS();
+}
+
+// Two sub-layers' outputs that read the same normalised rows: for output row i, r = rows ? rows[i] : i;
+// x = residual[r] + (first[r] + second[r]), all float; if store_residual: residual[r] = x;
+// out[i] = weight ? x / sqrt(mean(x^2) + eps) * weight : x.  A row a workgroup; the row is read once and kept in
+// registers (PER elements a thread, rows of up to 256 * PER).
+template <typename T, int PER>
+__global__ void __launch_bounds__(256)
+add_pair_rmsnorm_kernel(float* __restrict__ residual, const T* __restrict__ first, const T* __restrict__ second,
+                        const float* __restrict__ weight, T* __restrict__ out, const int* __restrict__ rows, int hidden,
+                        float eps, int store_residual) {
+  __shared__ float scratch[16];
+  const int i = blockIdx.x;
+  const int r = rows ? rows[i] : i;
+  float* res = residual + (size_t)r * hidden;
+  const T* a = first + (size_t)r * hidden;
+  const T* b = second + (size_t)r * hidden;
+  float x[PER];
+  float sq = 0.f;
+#pragma unroll
+  for (int p = 0; p < PER; ++p) {
+    const int h = p * 256 + threadIdx.x;
+    x[p] = 0.f;
+    if (h < hidden) {
+      x[p] = res[h] + (ld(a + h) + ld(b + h));
+      if (store_residual) res[h] = x[p];
+    }
+    sq += x[p] * x[p];
+  }
+  float inv = 1.f;
+  if (weight) inv = 1.0f / sqrtf(block_sum(sq, scratch) / (float)hidden + eps);
+  T* dst = out + (size_t)i * hidden;
+#pragma unroll
+  for (int p = 0; p < PER; ++p) {
+    const int h = p * 256 + threadIdx.x;
+    if (h < hidden) st(dst + h, weight ? x[p] * inv * weight[h] : x[p]);
+  }
+}
+
+extern "C" int ta_add_pair_rmsnorm(void* residual, const void* first, const void* second, const void* weight, void* out,
+                                   const void* rows, int n_rows, int hidden, float eps, int store_residual, int dtype,
+                                   hipStream_t stream) {
+  if (n_rows <= 0) return 0;
+  if (hidden <= 0 || hidden > 256 * 32 || !first || !second) return -1;
+#define PAIR(TT, PP) add_pair_rmsnorm_kernel<TT, PP><<<n_rows, 256, 0, stream>>>((float*)residual, (const TT*)first, \
+    (const TT*)second, (const float*)weight, (TT*)out, (const int*)rows, hidden, eps, store_residual)
+#define PAIR_SIZES(TT) if (hidden <= 256) PAIR(TT, 1); else if (hidden <= 1024) PAIR(TT, 4); else if (hidden <= 2048) PAIR(TT, 8); \
+                       else if (hidden <= 4096) PAIR(TT, 16); else PAIR(TT, 32)
+  if (dtype == DT_F32) { PAIR_SIZES(float); } else { PAIR_SIZES(bf16_t); }
+#undef PAIR_SIZES
+#undef PAIR
   return LAUNCH_STATUS();
 }
 

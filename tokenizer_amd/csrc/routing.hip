@@ -323,3 +323,191 @@ extern "C" int ta_gelu_gate(const void* in, void* out, int n_tokens, int inner, 
     gelu_gate_kernel<bf16_t><<<rt_blocks(total), 256, 0, stream>>>((const bf16_t*)in, (bf16_t*)out, inner, total);
   return LAUNCH_STATUS();
 }
+
+// ---------------------------------------------------------------------------------------------------------------
+// A router of sigmoid scores with a correction and groups, and experts without a gate branch.
+
+#define RS_MAX_EXPERTS 1024
+
+// logits: float [n_tokens, n_experts].  s = sigmoid(logit); an expert's choice score is s + correction.  With n_groups > 0
+// the experts form that many equal groups of neighbours; a group is worth the sum of its two largest choice scores (its
+// one score if it has one expert), and experts outside the `keep` best groups (the lower index of equals) count as minus
+// infinity.  The `top` largest choice scores (the lower index of equals) are chosen, in falling order; their weights
+// are their s over the sum of the chosen s (+ 1e-20).  A wave a token; the scores of a token lie in LDS.
+__global__ void __launch_bounds__(256)
+route_sigmoid_kernel(const float* __restrict__ logits, const float* __restrict__ correction, int n_tokens, int n_experts,
+                     int n_groups, int keep, int top, int* __restrict__ chosen, float* __restrict__ weights) {
+  extern __shared__ float rs_scratch[];
+  const int lane = threadIdx.x & (WAVE - 1), wave = threadIdx.x / WAVE;
+  const int slot = blockIdx.x * (blockDim.x / WAVE) + wave;
+  const bool live = slot < n_tokens;                          // (a wave past the end works on the last token and stores nothing)
+  const int t = live ? slot : n_tokens - 1;
+  float* choice = rs_scratch + (size_t)wave * (2 * n_experts + n_groups);
+  float* score = choice + n_experts;
+  float* worth = score + n_experts;
+  const float* row = logits + (size_t)t * n_experts;
+  for (int e = lane; e < n_experts; e += WAVE) {
+    const float s = 1.0f / (1.0f + expf(-row[e]));
+    score[e] = s;
+    choice[e] = s + correction[e];
+  }
+  __syncthreads();
+  if (n_groups > 0) {
+    const int per = n_experts / n_groups;
+    for (int g = lane; g < n_groups; g += WAVE) {
+      float first = -INFINITY, second = -INFINITY;
+      for (int i = 0; i < per; ++i) {
+        const float v = choice[g * per + i];
+        if (v > first) { second = first; first = v; }
+        else if (v > second) second = v;
+      }
+      worth[g] = per > 1 ? first + second : first;
+    }
+    __syncthreads();
+    for (int g = lane; g < n_groups; g += WAVE) {
+      const float mine = worth[g];
+      int ahead = 0;
+      for (int o = 0; o < n_groups; ++o) {
+        const float v = worth[o];
+        ahead += (v > mine || (v == mine && o < g)) ? 1 : 0;
+      }
+      if (ahead >= keep)
+        for (int i = 0; i < per; ++i) choice[g * per + i] = -INFINITY;
+    }
+    __syncthreads();
+  }
+  float total = 0.f, mine = 0.f;
+  int last = -1;
+  float last_value = INFINITY;
+  for (int k = 0; k < top; ++k) {
+    float best = -INFINITY;
+    int best_at = n_experts;
+    for (int e = lane; e < n_experts; e += WAVE) {
+      const float v = choice[e];
+      const bool behind = v < last_value || (v == last_value && e > last);
+      if (behind && (v > best || (v == best && e < best_at))) { best = v; best_at = e; }
+    }
+#pragma unroll
+    for (int off = WAVE / 2; off > 0; off >>= 1) {
+      const float other = __shfl_xor(best, off, WAVE);
+      const int other_at = __shfl_xor(best_at, off, WAVE);
+      if (other > best || (other == best && other_at < best_at)) { best = other; best_at = other_at; }
+    }
+    best_at = min(best_at, n_experts - 1);
+    const float s = score[best_at];
+    total += s;
+    if (lane == k) mine = s;
+    if (live && lane == 0) chosen[(size_t)t * top + k] = best_at;
+    last = best_at;
+    last_value = best;
+  }
+  if (live && lane < top) weights[(size_t)t * top + lane] = mine / (total + 1e-20f);
+}
+
+// up: [n_tokens, n_experts * inner]; out: [n_tokens, columns], columns >= n_experts * inner:
+// out[t, e * inner + i] = w * max(up, 0)^2 for an expert the token chose with weight w, 0 for the others and beyond.
+template <typename T>
+__global__ void expert_act_kernel(const T* __restrict__ up, const int* __restrict__ chosen, const float* __restrict__ weights,
+                                  int top, int n_experts, int inner, int columns, T* __restrict__ out, size_t total) {
+  const int in_stride = n_experts * inner;
+  for (size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += (size_t)gridDim.x * blockDim.x) {
+    const size_t t = idx / columns;
+    const int c = (int)(idx - t * columns);
+    float value = 0.f;
+    if (c < in_stride) {
+      const int e = c / inner;
+      float w = 0.f;
+      for (int k = 0; k < top; ++k)
+        if (chosen[t * top + k] == e) w += weights[t * top + k];
+      if (w != 0.f) {
+        const float z = fmaxf(ld(up + t * in_stride + c), 0.f);
+        value = w * (z * z);
+      }
+    }
+    st(out + idx, value);
+  }
+}
+
+// The same for bfloat16 rows in pieces of eight (inner and columns multiples of eight).
+__global__ void expert_act_vec_kernel(const bf16_t* __restrict__ up, const int* __restrict__ chosen,
+                                      const float* __restrict__ weights, int top, int n_experts, int inner, int columns,
+                                      bf16_t* __restrict__ out, size_t total8) {
+  const int in_stride = n_experts * inner, columns8 = columns / 8;
+  for (size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total8; idx += (size_t)gridDim.x * blockDim.x) {
+    const size_t t = idx / columns8;
+    const int c = (int)(idx - t * columns8) * 8;
+    float v[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    if (c < in_stride) {
+      const int e = c / inner;
+      float w = 0.f;
+      for (int k = 0; k < top; ++k)
+        if (chosen[t * top + k] == e) w += weights[t * top + k];
+      if (w != 0.f) {
+        rt_unpack8(*reinterpret_cast<const uint4*>(up + t * in_stride + c), v);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) { const float z = fmaxf(v[i], 0.f); v[i] = w * (z * z); }
+      }
+    }
+    *reinterpret_cast<uint4*>(out + idx * 8) = rt_pack8(v);
+  }
+}
+
+// out = max(in, 0)^2, element by element.
+template <typename T>
+__global__ void relu2_kernel(const T* __restrict__ in, T* __restrict__ out, size_t total) {
+  for (size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += (size_t)gridDim.x * blockDim.x) {
+    const float z = fmaxf(ld(in + idx), 0.f);
+    st(out + idx, z * z);
+  }
+}
+
+__global__ void relu2_vec_kernel(const bf16_t* __restrict__ in, bf16_t* __restrict__ out, size_t total8) {
+  for (size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total8; idx += (size_t)gridDim.x * blockDim.x) {
+    float v[8];
+    rt_unpack8(*reinterpret_cast<const uint4*>(in + idx * 8), v);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) { const float z = fmaxf(v[i], 0.f); v[i] = z * z; }
+    *reinterpret_cast<uint4*>(out + idx * 8) = rt_pack8(v);
+  }
+}
+
+extern "C" int ta_route_sigmoid(const void* logits, const void* correction, int n_tokens, int n_experts, int n_groups,
+                                int keep, int top, void* chosen, void* weights, hipStream_t stream) {
+  if (n_tokens <= 0) return 0;
+  if (top <= 0 || top > n_experts || top > WAVE || n_experts > RS_MAX_EXPERTS || n_groups < 0) return -1;
+  if (n_groups > 0 && (n_experts % n_groups || keep <= 0 || keep > n_groups || keep * (n_experts / n_groups) < top)) return -1;
+  const size_t lds = (size_t)4 * (2 * n_experts + n_groups) * sizeof(float);
+  route_sigmoid_kernel<<<(n_tokens + 3) / 4, 256, lds, stream>>>((const float*)logits, (const float*)correction, n_tokens,
+                                                                 n_experts, n_groups, keep, top, (int*)chosen, (float*)weights);
+  return LAUNCH_STATUS();
+}
+
+extern "C" int ta_expert_act(const void* up, const void* chosen, const void* weights, int n_tokens, int top, int n_experts,
+                             int inner, int columns, void* out, int dtype, hipStream_t stream) {
+  const size_t total = (size_t)n_tokens * columns;
+  if (total == 0) return 0;
+  if (columns < n_experts * inner) return -1;
+  if (dtype == DT_BF16 && inner % 8 == 0 && columns % 8 == 0 && (((uintptr_t)up | (uintptr_t)out) & 15) == 0) {
+    expert_act_vec_kernel<<<rt_blocks(total / 8), 256, 0, stream>>>((const bf16_t*)up, (const int*)chosen,
+        (const float*)weights, top, n_experts, inner, columns, (bf16_t*)out, total / 8);
+    return LAUNCH_STATUS();
+  }
+  if (dtype == DT_F32)
+    expert_act_kernel<float><<<rt_blocks(total), 256, 0, stream>>>((const float*)up, (const int*)chosen,
+        (const float*)weights, top, n_experts, inner, columns, (float*)out, total);
+  else
+    expert_act_kernel<bf16_t><<<rt_blocks(total), 256, 0, stream>>>((const bf16_t*)up, (const int*)chosen,
+        (const float*)weights, top, n_experts, inner, columns, (bf16_t*)out, total);
+  return LAUNCH_STATUS();
+}
+
+extern "C" int ta_relu2(const void* in, void* out, size_t total, int dtype, hipStream_t stream) {
+  if (total == 0) return 0;
+  if (dtype == DT_BF16 && total % 8 == 0 && (((uintptr_t)in | (uintptr_t)out) & 15) == 0)
+    relu2_vec_kernel<<<rt_blocks(total / 8), 256, 0, stream>>>((const bf16_t*)in, (bf16_t*)out, total / 8);
+  else if (dtype == DT_F32)
+    relu2_kernel<float><<<rt_blocks(total), 256, 0, stream>>>((const float*)in, (float*)out, total);
+  else
+    relu2_kernel<bf16_t><<<rt_blocks(total), 256, 0, stream>>>((const bf16_t*)in, (bf16_t*)out, total);
+  return LAUNCH_STATUS();
+}

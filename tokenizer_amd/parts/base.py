@@ -213,6 +213,22 @@ class NormedDelta:
         return self.ops.norm_add_rmsnorm(zero, self.rows, self.weight, self.eps, None, 0.0, out, store_residual=False)
 
 
+class SumDelta:
+    """What a layer whose two sub-layers read the same normalised rows hands on: their outputs `first` and `second`
+    [T, H] (compute dtype), still to be added to each other and to the stream, x + (first + second) in float32.  A norm
+    of the form x / sqrt(mean(x^2) + eps) * w takes it as its delta and does the two additions and the norm in one
+    kernel (`ops.add_pair_rmsnorm`); for anyone else `resolve()` gives the sum as a float32 tensor."""
+
+    def __init__(self, ops, first: torch.Tensor, second: torch.Tensor):
+        self.ops, self.first, self.second = ops, first, second
+
+    def resolve(self) -> torch.Tensor:
+        zero = torch.zeros(self.first.shape, dtype=torch.float32, device=self.first.device)
+        rows = torch.empty(self.first.shape, dtype=self.first.dtype, device=self.first.device)
+        self.ops.add_pair_rmsnorm(zero, self.first, self.second, None, 0.0, rows)
+        return zero
+
+
 def as_tensor(delta):
     """The delta as a tensor: a product still in parts has them added now."""
     resolve = getattr(delta, "resolve", None)

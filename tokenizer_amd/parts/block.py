@@ -3,7 +3,7 @@ from __future__ import annotations
 
 import torch
 
-from .base import BLOCKS, Block, NormedDelta, Repeatable, as_tensor, repeatable_of
+from .base import BLOCKS, Block, NormedDelta, Repeatable, SumDelta, as_tensor, repeatable_of
 from .spec import TensorSpec
 
 
@@ -36,6 +36,28 @@ class PreNormBlock(Block):
         if self.feed_forward is not None:
             delta = self.feed_forward.forward_normed(residual, delta, self.feed_forward_norm, ctx)
         return delta
+
+
+@BLOCKS.register("parallel")
+class ParallelBlock(Block):
+    """x + (mixer(h) + feed_forward(h)) with h = norm(x): one norm, and both sub-layers read its output.  The mixer's
+    norm is the layer's norm (a feed-forward norm in the layer's spec names the same tensor and is not used).  The two
+    outputs are handed on together (`SumDelta`): the next layer's norm adds them to each other and to the float32
+    stream and normalises the sum in one kernel.  A layer without a feed-forward hands the mixer's output on alone."""
+    graph_safe = True
+
+    def __init__(self, mixer_norm, mixer, feed_forward_norm, feed_forward):
+        if mixer is None:
+            raise ValueError("a parallel layer has a mixer; its norm is the layer's norm")
+        self.mixer_norm, self.mixer = mixer_norm, mixer
+        self.feed_forward_norm, self.feed_forward = feed_forward_norm, feed_forward
+
+    def forward(self, residual, delta, ctx, cache):
+        h = self.mixer_norm.apply(residual, delta)
+        mixed = self.mixer.forward(h, ctx, cache)
+        if self.feed_forward is None:
+            return mixed
+        return SumDelta(self.mixer.runtime.ops, mixed, self.feed_forward.forward(h, ctx))
 
 
 @BLOCKS.register("sandwich_norm")

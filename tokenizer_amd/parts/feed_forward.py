@@ -102,23 +102,44 @@ class RoutedExperts(FeedForward):
     that belong to one expert each, multiply every tile with its expert's matrices alone, and add a token's experts
     up at the end (the shared expert runs as a dense one).  Either way the routing stays on the device, so the step's
     launches do not depend on it.
+
+    Two options of the spec change what an expert and the router are, each on its own.  `gated` False: an expert is
+    down(act(up(x))) with tensors `e<j>.up|down` alone, and `activation` "relu2" is max(z, 0)^2; all experts' up
+    matrices are one matrix, and the kernel between the two products leaves weight * act(up) for chosen experts and
+    zero for the others.  `router` "sigmoid": scores s = sigmoid(logit); an expert's choice score is s + `correction`
+    (a tensor, one number an expert); with `n_groups` the experts form that many equal groups of neighbours, a group is
+    worth the sum of its two largest choice scores, and only experts of the `keep_groups` best groups can be chosen
+    (the others count as minus infinity); the `top_k` largest choice scores are chosen and weighted by their s over
+    the chosen's sum (+ 1e-20).  Logits, scores and weights are float32.
     """
     graph_safe = True
     GROUPED_FROM = 1024        # (token, expert) pairs from which the sorted form runs
 
     def __init__(self, spec: FeedForwardSpec, tensors: dict[str, torch.Tensor], runtime: Runtime):
-        if spec.activation != "silu":
-            raise ValueError(f"routed_experts knows the activation silu, not {spec.activation!r}")
+        if (spec.activation, spec.gated) not in (("silu", True), ("relu2", False)):
+            raise ValueError(f"routed_experts knows gated silu experts and ungated relu2 experts, not "
+                             f"{'gated' if spec.gated else 'ungated'} {spec.activation!r}")
         if not 0 < spec.top_k <= spec.n_experts:
             raise ValueError(f"{spec.top_k} of {spec.n_experts} experts")
+        if spec.router not in ("softmax", "sigmoid"):
+            raise ValueError(f"router {spec.router!r}: known are softmax and sigmoid")
         self.spec, self.runtime = spec, runtime
         self.n_experts, self.top_k = spec.n_experts, spec.top_k
         self.inner, self.shared = spec.intermediate_size, spec.shared_size
+        self.gated, self.sigmoid = spec.gated, spec.router == "sigmoid"
+        if not self.gated and self.shared:
+            raise ValueError("ungated experts have no shared expert here")
         self.w_router = tensors["router"]
+        if self.sigmoid:
+            self.correction = tensors["correction"].to(torch.float32).contiguous()
+            self.n_groups, self.keep_groups = int(spec.n_groups), int(spec.keep_groups)
+            if self.n_groups and (self.n_experts % self.n_groups or not 0 < self.keep_groups <= self.n_groups
+                                  or self.keep_groups * (self.n_experts // self.n_groups) < self.top_k):
+                raise ValueError(f"{self.n_groups} groups of {self.n_experts} experts, {self.keep_groups} kept, {self.top_k} a token")
         names = [f"e{j}" for j in range(self.n_experts)] + (["shared"] if self.shared else [])
         gate_up, down = [], []
         for name in names:
-            gate_up += [tensors[f"{name}.gate"], tensors[f"{name}.up"]]
+            gate_up += [tensors[f"{name}.gate"], tensors[f"{name}.up"]] if self.gated else [tensors[f"{name}.up"]]
             down.append(tensors[f"{name}.down"])
         self.total = self.n_experts * self.inner + self.shared           # columns between the two products
         fill = (-self.total) % 8 if runtime.dtype == torch.bfloat16 else 0     # the second product reads K in eights
@@ -138,26 +159,36 @@ class RoutedExperts(FeedForward):
     @staticmethod
     def tensor_specs(spec: FeedForwardSpec) -> dict[str, TensorSpec]:
         out = {"router": TensorSpec((spec.n_experts, spec.hidden_size), std=0.5)}
+        if spec.router == "sigmoid":
+            out["correction"] = TensorSpec((spec.n_experts,), role="vector", std=0.2)
         sizes = [(f"e{j}", spec.intermediate_size) for j in range(spec.n_experts)]
         if spec.shared_size:
             sizes.append(("shared", spec.shared_size))
         for name, inner in sizes:
-            out.update({f"{name}.gate": TensorSpec((inner, spec.hidden_size)), f"{name}.up": TensorSpec((inner, spec.hidden_size)),
-                        f"{name}.down": TensorSpec((spec.hidden_size, inner))})
+            if spec.gated:
+                out[f"{name}.gate"] = TensorSpec((inner, spec.hidden_size))
+            out.update({f"{name}.up": TensorSpec((inner, spec.hidden_size)), f"{name}.down": TensorSpec((spec.hidden_size, inner))})
         return out
 
     def forward(self, x, ctx):
         ops = self.runtime.ops
         chosen = torch.empty((x.shape[0], self.top_k), dtype=torch.int32, device=x.device)
         weights = torch.empty((x.shape[0], self.top_k), dtype=torch.float32, device=x.device)
-        fused = getattr(ops, "route_rows", None)          # the router's product and the choice in one kernel, where there is one
-        if fused is None or not fused(x, self.w_router, chosen, weights):
-            ops.route_top(ops.linear(x, self.w_router, out_dtype=torch.float32), chosen, weights)
+        if self.sigmoid:
+            ops.route_sigmoid(ops.linear(x, self.w_router, out_dtype=torch.float32), self.correction, self.n_groups,
+                              self.keep_groups, chosen, weights)
+        else:
+            fused = getattr(ops, "route_rows", None)      # the router's product and the choice in one kernel, where there is one
+            if fused is None or not fused(x, self.w_router, chosen, weights):
+                ops.route_top(ops.linear(x, self.w_router, out_dtype=torch.float32), chosen, weights)
         if self.groupable and x.shape[0] * self.top_k >= self.GROUPED_FROM and hasattr(ops, "grouped_linear"):
             return self._sorted(x, chosen, weights)
         gate_up = ops.linear(x, self.w_gate_up)
         act = torch.empty((x.shape[0], self.columns), dtype=x.dtype, device=x.device)
-        ops.expert_gate(gate_up, chosen, weights, self.n_experts, self.inner, self.shared, act)
+        if self.gated:
+            ops.expert_gate(gate_up, chosen, weights, self.n_experts, self.inner, self.shared, act)
+        else:
+            ops.expert_act(gate_up, chosen, weights, self.n_experts, self.inner, act)
         return ops.linear(act, self.w_down)
 
     def _sorted(self, x, chosen, weights):
@@ -166,10 +197,13 @@ class RoutedExperts(FeedForward):
         hidden, inner = x.shape[1], self.inner
         bm = 128 if x.shape[0] * self.top_k >= 2048 * max(1, self.n_experts // 8) else 64
         slot_of, row_of, tile_expert = ops.expert_slots(chosen, self.n_experts, bm)
-        gate_up = ops.grouped_linear(x, row_of, tile_expert, bm, self.w_gate_up, 2 * inner * hidden, 2 * inner, hidden,
-                                     torch.bfloat16)
+        wide = (2 if self.gated else 1) * inner          # an expert's rows of the joined first matrix
+        gate_up = ops.grouped_linear(x, row_of, tile_expert, bm, self.w_gate_up, wide * hidden, wide, hidden, torch.bfloat16)
         act = torch.empty((gate_up.shape[0], inner), dtype=x.dtype, device=x.device)
-        ops.silu_gate(gate_up, act)
+        if self.gated:
+            ops.silu_gate(gate_up, act)
+        else:
+            ops.relu2(gate_up, act)
         rows = ops.grouped_linear(act, None, tile_expert, bm, self.w_down, inner, hidden, inner, torch.float32)
         shared = None
         if self.shared:

@@ -230,6 +230,8 @@ class DecoderModel:
     def embed(self, ctx) -> torch.Tensor:
         """The float32 residual stream [tokens, hidden] the first layer starts from."""
         residual = torch.empty((ctx.n_tokens, self.spec.hidden_size), dtype=torch.float32, device=self.runtime.device)
+        if self.spec.embedding_scale != 1.0:
+            return self.runtime.ops.embedding(ctx.token_ids, self.embedding, residual, scale=float(self.spec.embedding_scale))
         return self.runtime.ops.embedding(ctx.token_ids, self.embedding, residual)
 
     def logits(self, residual: torch.Tensor, delta, ctx) -> torch.Tensor:

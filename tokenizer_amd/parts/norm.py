@@ -3,7 +3,7 @@ from __future__ import annotations
 
 import torch
 
-from .base import NORMS, Norm, NormedDelta, NormFold, Repeatable, Runtime
+from .base import NORMS, Norm, NormedDelta, NormFold, Repeatable, Runtime, SumDelta
 from .spec import NormSpec, TensorSpec
 
 
@@ -11,14 +11,19 @@ from .spec import NormSpec, TensorSpec
 class RMSNorm(Norm):
     """y = x / sqrt(mean(x^2) + eps) * weight (qwen-infer/src/model.rs:594-599), in float32.  The weight is the
     tensor `weight` under the norm's prefix, or (option `tensor_name`) another name there; the empty name is the
-    tensor that the prefix itself names.  A delta that is itself still to be normalised (`NormedDelta`) is
-    normalised, scaled and added in the same kernel."""
+    tensor that the prefix itself names.  Option `offset` c: the stored tensor lies around zero and the scale is
+    c + weight (formed once, in float32).  A delta that is itself still to be normalised (`NormedDelta`) is
+    normalised, scaled and added in the same kernel; so are the two terms of a `SumDelta` (two sub-layers that read
+    the same normalised rows)."""
     graph_safe = True
 
 
     def __init__(self, spec: NormSpec, tensors: dict[str, torch.Tensor], runtime: Runtime):
         self.size, self.eps = spec.size, float(spec.eps)
         self.weight = tensors[spec.options.get("tensor_name", "weight")]
+        offset = float(spec.options.get("offset") or 0.0)
+        if offset:
+            self.weight = (self.weight.to(torch.float32) + offset).contiguous()
         self.runtime = runtime
 
     @staticmethod
@@ -34,6 +39,9 @@ class RMSNorm(Norm):
     def apply(self, residual, delta, rows=None):
         n_rows = residual.shape[0] if rows is None else rows.numel()
         out = torch.empty((n_rows, self.size), dtype=self.runtime.dtype, device=residual.device)
+        if isinstance(delta, SumDelta):
+            return self.runtime.ops.add_pair_rmsnorm(residual, delta.first, delta.second, self.weight, self.eps, out, rows,
+                                                     store_residual=rows is None)
         if isinstance(delta, NormedDelta):
             if delta.side is not None:
                 done = delta.side.fused(residual, delta, self.weight, self.eps, out, rows)

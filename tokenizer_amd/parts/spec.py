@@ -21,11 +21,21 @@ class TensorSpec:
     feed matrix products and are held in the compute dtype, "vector" tensors
     (norm scales, biases) are small and held in float32, "table" tensors are
     integer tables kept as int32, "keep" tensors stay as the file stores them.
+    A -1 in `shape` is a size that only the file gives (no configuration key names it): the loader takes what it
+    finds there, and the random-weights mode writes `free_size`.
     """
     shape: tuple[int, ...]
     init: str = "normal"
     std: float = 0.02
     role: str = "matrix"
+    free_size: int = 0
+
+    def fits(self, shape) -> bool:
+        shape = tuple(shape)
+        return len(shape) == len(self.shape) and all(want in (-1, found) for want, found in zip(self.shape, shape))
+
+    def drawn_shape(self) -> tuple[int, ...]:
+        return tuple(self.free_size if size == -1 else size for size in self.shape)
 
 
 @dataclasses.dataclass(frozen=True)
@@ -110,6 +120,13 @@ class MixerSpec:
     #                               lambda = exp(lq1.lk1) - exp(lq2.lk2) + c, o brought to unit RMS per head, times 1 - c
     qk_norm: str | None = None    # "whole": RMS norm with a weight over all query rows at once (and all key rows), before rotation
     head_gate: bool = False       # each head's output times sigmoid of one number projected from the mixer's input
+    q_rank: int = 0               # latent attention: width of the normalised latent the queries are projected up from
+    kv_rank: int = 0              # latent attention: width of the normalised latent that keys and values are projected
+    #                               up from (the latent is what the cache keeps, with the rotated key part behind it)
+    rot_dim: int = 0              # latent attention: coordinates at the end of every query head that are rotated and meet
+    #                               one rotated key part shared by all heads (0: no positions at all)
+    element_gate: bool = False    # the mixer's output times sigmoid of a projection of its input, coordinate by coordinate
+    conv_taps: int = 0            # recurrent mixers: taps of the short causal convolution over q, k and v (0: none)
     tensor_names: tuple[tuple[str, str], ...] = ()   # (part's name, file's name) where a file names tensors otherwise
     options: dict[str, Any] = dataclasses.field(default_factory=dict, hash=False, compare=False)
 
@@ -126,6 +143,13 @@ class FeedForwardSpec:
     n_experts: int = 0            # routed feed-forwards: experts of `intermediate_size`, of which a token uses `top_k`
     top_k: int = 0
     shared_size: int = 0          # inner width of an expert that every token uses (0: none)
+    gated: bool = True            # experts are down(act(gate) * up); False: down(act(up)), tensors `up` and `down` alone
+    router: str = "softmax"       # "softmax": the largest logits, weighted by the softmax over the chosen; "sigmoid":
+    #                               scores s = sigmoid(logit), chosen by s + `correction` (a tensor, one number an
+    #                               expert), weighted by s over the chosen's sum
+    n_groups: int = 0             # "sigmoid": experts form so many equal groups of neighbours (0: no groups) ...
+    keep_groups: int = 0          # ... of which only the best so many (by the sum of a group's two largest choice
+    #                               scores) can be chosen from
     tensor_names: tuple[tuple[str, str], ...] = ()
     options: dict[str, Any] = dataclasses.field(default_factory=dict, hash=False, compare=False)
 
@@ -192,6 +216,7 @@ class ModelSpec:
     tied_head: bool
     head_name: str                # used when the head is not tied
     embedding_std: float = 0.02
+    embedding_scale: float = 1.0  # the embedding's rows are multiplied by this on their way into the stream
     frame: str = "decoder"        # what stands around the layers (`parts.base.FRAMES`)
     extra_cache_units: tuple[int, ...] = ()   # cache unit n_layers + i repeats the need of layer extra_cache_units[i]
     options: dict[str, Any] = dataclasses.field(default_factory=dict, hash=False, compare=False)   # the frame's own constants

@@ -145,7 +145,7 @@ def load_weights(folder: str, expected: dict[str, TensorSpec], compute_dtype: to
     for name in sorted(names & set(expected)):
         shape, dtype = source.info(name)
         spec = expected[name]
-        if tuple(shape) != tuple(spec.shape):
+        if not spec.fits(shape):
             wrong_shape.append((name, shape, spec.shape))
         if spec.role in ("matrix", "vector") and dtype not in _FLOATS:
             wrong_dtype.append((name, dtype))

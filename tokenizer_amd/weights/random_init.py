@@ -27,6 +27,9 @@ def _generator(seed: int, name: str) -> torch.Generator:
 
 
 def random_tensor(name: str, spec: TensorSpec, seed: int, norm_spread: float = 0.0) -> torch.Tensor:
+    if -1 in spec.shape:                   # a size no configuration key names: the spec's own choice
+        import dataclasses
+        spec = dataclasses.replace(spec, shape=spec.drawn_shape())
     if spec.role == "table":
         return torch.zeros(spec.shape, dtype=torch.int32)
     if spec.init == "ones":
