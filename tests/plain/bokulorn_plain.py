@@ -198,3 +198,13 @@ def forward(cfg: dict, tensors: dict, ids: list[int], layers_out: list | None = 
         if layers_out is not None:
             layers_out.append(x.clone())
     return offset_norm(x, tensors["final.norm"], eps) @ tensors["head"].T
+
+
+def greedy_generate(cfg: dict, tensors: dict, prompt, n_new: int) -> list[int]:
+    """The first maximum of the last position's logits, appended and run again from the start, `n_new` times."""
+    ids, out = list(prompt), []
+    for _ in range(n_new):
+        logits = forward(cfg, tensors, ids)[-1]
+        out.append(int(torch.argmax(logits)))
+        ids.append(out[-1])
+    return out

@@ -155,7 +155,9 @@ class Ops:
                      "ta_sample_workspace_words", "ta_library_gemm_bf16", "ta_compute_units", "ta_read_stream",
                      "ta_embedding_streams", "ta_streams_step", "ta_token_shift", "ta_mlstm_scan", "ta_mlstm_chunked", "ta_head_norm_gate",
                      "ta_capped_gate", "ta_norm_add_rmsnorm", "ta_norm_rotate_store", "ta_differential_heads",
-                     "ta_sigmoid_head_gate", "ta_route_top", "ta_expert_gate", "ta_side_gate", "ta_gelu_gate", "ta_norm_side_norm", "ta_route_rows", "ta_expert_slots", "ta_grouped_gemm_bf16", "ta_expert_combine"):
+                     "ta_sigmoid_head_gate", "ta_route_top", "ta_expert_gate", "ta_side_gate", "ta_gelu_gate", "ta_norm_side_norm", "ta_route_rows", "ta_expert_slots", "ta_grouped_gemm_bf16", "ta_expert_combine",
+                     "ta_add_pair_rmsnorm", "ta_latent_store", "ta_rotate_tails", "ta_head_linear", "ta_short_conv_silu",
+                     "ta_delta_scan", "ta_route_sigmoid", "ta_expert_act", "ta_relu2"):
             getattr(self.lib, name).restype = ctypes.c_int
         self.lib.ta_grouped_gemm_bf16.argtypes = [ctypes.c_void_p, ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int,
                                                   ctypes.c_int, ctypes.c_void_p, ctypes.c_long, ctypes.c_int, ctypes.c_void_p,
@@ -220,14 +222,14 @@ class Ops:
         return out
 
     # ------------------------------------------------------------------ embedding
-    def embedding(self, ids: torch.Tensor, table: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
-        """out[t] = table[ids[t]] as float32.  ids int32 [T]; table [V, H]; out float32 [T, H]."""
+    def embedding(self, ids: torch.Tensor, table: torch.Tensor, out: torch.Tensor, scale: float = 1.0) -> torch.Tensor:
+        """out[t] = table[ids[t]] * scale as float32.  ids int32 [T]; table [V, H]; out float32 [T, H]."""
         _dev(ids, table, out)
         n, (vocab, hidden) = ids.numel(), table.shape
         _need(ids.dtype == torch.int32 and ids.dim() == 1, "ids must be int32 [T]")
         _need(out.dtype == torch.float32 and tuple(out.shape) == (n, hidden), "out must be float32 [T, H]")
         self._check(self.lib.ta_embedding(_ptr(ids), _ptr(table), _ptr(out), n, hidden, vocab,
-                                          _code(table.dtype), self._stream()), "embedding")
+                                          _code(table.dtype), ctypes.c_float(scale), self._stream()), "embedding")
         return out
 
     # ---------------------------------------------------------------------- norm
@@ -269,6 +271,196 @@ class Ops:
         self._check(self.lib.ta_add_rmsnorm(_ptr(residual), _ptr(delta), _ptr(weight), _ptr(out), _ptr(rows),
                                             n_rows, hidden, ctypes.c_float(eps), int(store_residual),
                                             _code(out.dtype), self._stream()), "add_rmsnorm")
+        return out
+
+    def add_pair_rmsnorm(self, residual: torch.Tensor, first: torch.Tensor, second: torch.Tensor,
+                         weight: torch.Tensor | None, eps: float, out: torch.Tensor, rows: torch.Tensor | None = None,
+                         store_residual: bool = True) -> torch.Tensor:
+        """x = residual[r] + (first[r] + second[r]) in float32; optionally residual[r] = x; out[i] = rmsnorm(x) * weight
+        (weight None: out[i] = x).  residual float32 [T, H]; first, second [T, H] in out's dtype; weight float32 [H];
+        rows int32 [R] picks the rows (None: all); out [R, H]."""
+        _dev(residual, first, second, weight, out, rows)
+        n_tokens, hidden = residual.shape
+        n_rows = n_tokens if rows is None else rows.numel()
+        _need(residual.dtype == torch.float32, "the residual stream is float32")
+        _need(weight is None or (weight.dtype == torch.float32 and weight.numel() == hidden), "norm weight must be float32 [H]")
+        _need(tuple(first.shape) == (n_tokens, hidden) == tuple(second.shape) and first.dtype == out.dtype == second.dtype,
+              "the two terms are [T, H] in the output's dtype")
+        _need(tuple(out.shape) == (n_rows, hidden), "norm output has the wrong shape")
+        _need(rows is None or (rows.dtype == torch.int32 and not store_residual), "rows int32, and a subset stores nothing back")
+        _need(hidden <= 8192, "rows of up to 8192 elements")
+        self._check(self.lib.ta_add_pair_rmsnorm(_ptr(residual), _ptr(first), _ptr(second), _ptr(weight), _ptr(out), _ptr(rows),
+                                                 n_rows, hidden, ctypes.c_float(eps), int(bool(store_residual)),
+                                                 _code(out.dtype), self._stream()), "add_pair_rmsnorm")
+        return out
+
+    # ---------------------------------------------------- attention over a cached latent
+    def latent_store(self, rows: torch.Tensor, q_offset: int, q_rank: int, q_norm: torch.Tensor, kv_offset: int, kv_rank: int,
+                     kv_norm: torch.Tensor, rot_dim: int, rates: torch.Tensor | None, eps: float, positions: torch.Tensor,
+                     slots: torch.Tensor | None, k_pages: torch.Tensor | None, v_pages: torch.Tensor | None,
+                     latent_q: torch.Tensor) -> None:
+        """latent_q[t] = rmsnorm(rows[t, q_offset : + q_rank]) * q_norm; the kept row of a token, [rmsnorm(rows[t,
+        kv_offset : + kv_rank]) * kv_norm | the rot_dim coordinates behind them, coordinate i with i + rot_dim / 2 turned by
+        positions[t] * rates[i]], goes into key pages [n_pages, 1, page_size, kv_rank + rot_dim] at slots[t] and,
+        transposed within a page, into value pages [n_pages, 1, kv_rank + rot_dim, page_size] (slots None: nothing is
+        stored).  Norms and angles are float32."""
+        _dev(rows, q_norm, kv_norm, rates, positions, slots, k_pages, v_pages, latent_q)
+        n_tokens = rows.shape[0]
+        _need(rows.dim() == 2 and q_offset >= 0 and kv_offset >= 0 and q_offset + q_rank <= rows.shape[1]
+              and kv_offset + kv_rank + rot_dim <= rows.shape[1] and q_rank > 0 and kv_rank > 0, "the latents do not fit the rows")
+        _need(q_norm.dtype == torch.float32 and q_norm.numel() == q_rank and kv_norm.dtype == torch.float32
+              and kv_norm.numel() == kv_rank, "the latents' norm weights are float32")
+        _need(rot_dim >= 0 and rot_dim % 2 == 0 and (rot_dim == 0 or (rates is not None and rates.dtype == torch.float32
+                                                                       and rates.numel() == rot_dim // 2)),
+              "a rotation has an even number of coordinates and a float32 rate for each pair")
+        _need(positions.dtype == torch.int32 and positions.numel() == n_tokens, "positions must be int32 [T]")
+        _need(tuple(latent_q.shape) == (n_tokens, q_rank) and latent_q.dtype == rows.dtype, "latent_q is [T, q_rank]")
+        page_size = 0
+        if slots is not None:
+            _need(slots.dtype == torch.int32 and slots.numel() == n_tokens, "slots must be int32 [T]")
+            _need(k_pages is not None and v_pages is not None and k_pages.dtype == rows.dtype == v_pages.dtype,
+                  "pages must have the rows' dtype")
+            page_size = self._page_size(k_pages, v_pages, 1, kv_rank + rot_dim)
+        self._check(self.lib.ta_latent_store(_ptr(rows), rows.shape[1], q_offset, q_rank, _ptr(q_norm), kv_offset, kv_rank,
+                                             _ptr(kv_norm), rot_dim, _ptr(rates), ctypes.c_float(eps), _ptr(positions),
+                                             _ptr(slots), _ptr(k_pages if slots is not None else None),
+                                             _ptr(v_pages if slots is not None else None), page_size, _ptr(latent_q),
+                                             n_tokens, _code(rows.dtype), self._stream()), "latent_store")
+
+    def head_linear(self, x: torch.Tensor, x_offset: int, x_head_stride: int, weight: torch.Tensor, out: torch.Tensor,
+                    out_offset: int, out_head_stride: int) -> torch.Tensor:
+        """Products head by head: out[t, h out_head_stride + out_offset + n] = sum_k x[t, h x_head_stride + x_offset + k]
+        weight[h, n, k]; weight [heads, N, K]; float32 sums.  Other columns of `out` are left as they are."""
+        _dev(x, weight, out)
+        _need(weight.dim() == 3 and x.dim() == 2 and out.dim() == 2 and x.dtype == weight.dtype == out.dtype,
+              "x [T, .], weight [heads, N, K], out [T, .] of one dtype")
+        heads, n, k = weight.shape
+        m = x.shape[0]
+        _need(out.shape[0] == m and x_offset >= 0 and out_offset >= 0 and heads > 0
+              and (heads - 1) * x_head_stride + x_offset + k <= x.shape[1]
+              and (heads - 1) * out_head_stride + out_offset + n <= out.shape[1], "the heads do not fit the rows")
+        self._check(self.lib.ta_head_linear(_ptr(x), x.shape[1], x_head_stride, x_offset, _ptr(weight), _ptr(out), out.shape[1],
+                                            out_head_stride, out_offset, m, n, k, heads, _code(x.dtype), self._stream()),
+                    "head_linear")
+        return out
+
+    def rotate_tails(self, q: torch.Tensor, heads: int, head_width: int, tail_offset: int, dims: int, rates: torch.Tensor,
+                     positions: torch.Tensor, out: torch.Tensor, out_head_stride: int, out_offset: int) -> torch.Tensor:
+        """out[t, h out_head_stride + out_offset + i], i < dims: coordinates tail_offset.. of head h of q [T, heads
+        head_width], coordinate i with i + dims / 2 turned by positions[t] * rates[i] (float32 angles)."""
+        _dev(q, rates, positions, out)
+        n_tokens = q.shape[0]
+        _need(q.shape[1] >= heads * head_width and tail_offset >= 0 and tail_offset + dims <= head_width and dims % 2 == 0,
+              "the tails do not fit the heads")
+        _need(rates.dtype == torch.float32 and rates.numel() == dims // 2, "a float32 rate for each pair")
+        _need(positions.dtype == torch.int32 and positions.numel() == n_tokens, "positions must be int32 [T]")
+        _need(out.shape[0] == n_tokens and out.dtype == q.dtype and out_offset >= 0
+              and (heads - 1) * out_head_stride + out_offset + dims <= out.shape[1], "the tails do not fit the output")
+        self._check(self.lib.ta_rotate_tails(_ptr(q), q.shape[1], heads, head_width, tail_offset, dims, _ptr(rates),
+                                             _ptr(positions), _ptr(out), out.shape[1], out_head_stride, out_offset, n_tokens,
+                                             _code(q.dtype), self._stream()), "rotate_tails")
+        return out
+
+    # ---------------------------------------------------- delta rule with a decay per key channel
+    def short_conv_silu(self, rows: torch.Tensor, offsets, widths, taps: torch.Tensor, state: torch.Tensor, state_offset: int,
+                        cu_q: torch.Tensor, first_position: torch.Tensor, state_slots: torch.Tensor,
+                        entry_of_token: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+        """A short causal convolution over time, channel by channel, then silu.  The channels are up to three runs of
+        columns of `rows` (run i: widths[i] columns from offsets[i] on), side by side in `out` [T, channels]; taps float32
+        [channels, n_taps], the last column the current token's.  Inputs before an entry's first row are its state row's
+        [state_offset : + (n_taps - 1) channels] (oldest first; zeros if its first position is 0), which then takes the
+        entry's last n_taps - 1 inputs."""
+        _dev(rows, taps, state, cu_q, first_position, state_slots, entry_of_token, out)
+        offsets, widths = [int(o) for o in offsets], [int(w) for w in widths]
+        _need(len(offsets) == len(widths) and 1 <= len(widths) <= 3, "one to three runs of channels")
+        while len(widths) < 3:
+            offsets.append(0)
+            widths.append(0)
+        channels, n_tokens = sum(widths), rows.shape[0]
+        _need(all(w >= 0 and o >= 0 and o + w <= rows.shape[1] for o, w in zip(offsets, widths)), "the runs do not fit the rows")
+        _need(taps.dtype == torch.float32 and taps.dim() == 2 and taps.shape[0] == channels and 1 <= taps.shape[1] <= 16,
+              "taps float32 [channels, up to 16]")
+        n_taps = taps.shape[1]
+        _need(state.dtype == torch.float32 and state.dim() == 2 and state.shape[1] >= state_offset + (n_taps - 1) * channels,
+              "state rows are too short")
+        _need(tuple(out.shape) == (n_tokens, channels) and out.dtype == rows.dtype and entry_of_token.numel() == n_tokens,
+              "out is [T, channels]")
+        n_entries = cu_q.numel() - 1
+        _need(first_position.numel() == n_entries == state_slots.numel(), "one first position and slot per entry")
+        self._check(self.lib.ta_short_conv_silu(_ptr(rows), rows.shape[1], offsets[0], widths[0], offsets[1], widths[1],
+                                                offsets[2], widths[2], _ptr(taps), n_taps, _ptr(state),
+                                                ctypes.c_long(state.shape[1]), state_offset, _ptr(cu_q), _ptr(first_position),
+                                                _ptr(state_slots), _ptr(entry_of_token), _ptr(out), n_tokens, n_entries,
+                                                _code(rows.dtype), self._stream()), "short_conv_silu")
+        return out
+
+    def delta_scan(self, fresh: torch.Tensor, decay: torch.Tensor, neg_rate: torch.Tensor, rows: torch.Tensor, beta_offset: int,
+                   state: torch.Tensor, cu_q: torch.Tensor, first_position: torch.Tensor, state_slots: torch.Tensor,
+                   out: torch.Tensor, heads: int, groups: int, d: int, dv: int, unit_eps: float) -> torch.Tensor:
+        """The gated delta rule over every entry's rows, from and into the entries' state rows.
+
+        fresh [T, 2 groups d + heads dv]: q, k (groups of d; head h reads group h // (heads / groups)) and v (heads of
+        dv); q and k become unit vectors, x / sqrt(sum x^2 + unit_eps), q times d^(-1/2).  decay float32 [T, heads d]:
+        g = exp(neg_rate[h] * softplus(decay)); beta = sigmoid(rows[t, beta_offset + h]).  Per head and token:
+        S <- diag(g) S; u = beta (v - S^T k); S <- S + k u^T; out = S^T q.  state float32 [slots, >= heads d dv] (an
+        entry whose first position is 0 starts from zeros); out float32 [T, heads dv]."""
+        _dev(fresh, decay, neg_rate, rows, state, cu_q, first_position, state_slots, out)
+        n_tokens = fresh.shape[0]
+        _need(heads > 0 and groups > 0 and heads % groups == 0 and 0 < d <= 256 and dv > 0, "heads of up to 256 key channels")
+        _need(fresh.shape[1] == 2 * groups * d + heads * dv, "q, k, v do not fit the rows")
+        _need(decay.dtype == torch.float32 and tuple(decay.shape) == (n_tokens, heads * d), "decay float32 [T, heads d]")
+        _need(neg_rate.dtype == torch.float32 and neg_rate.numel() == heads, "neg_rate float32 [heads]")
+        _need(rows.shape[0] == n_tokens and rows.dtype == fresh.dtype and 0 <= beta_offset and beta_offset + heads <= rows.shape[1],
+              "beta does not fit the rows")
+        _need(state.dtype == torch.float32 and state.dim() == 2 and state.shape[1] >= heads * d * dv, "state rows are too short")
+        _need(out.dtype == torch.float32 and tuple(out.shape) == (n_tokens, heads * dv), "out float32 [T, heads dv]")
+        n_entries = cu_q.numel() - 1
+        _need(first_position.numel() == n_entries == state_slots.numel(), "one first position and slot per entry")
+        self._check(self.lib.ta_delta_scan(_ptr(fresh), fresh.shape[1], _ptr(decay), _ptr(neg_rate), _ptr(rows), rows.shape[1],
+                                           beta_offset, _ptr(state), ctypes.c_long(state.shape[1]), _ptr(cu_q),
+                                           _ptr(first_position), _ptr(state_slots), _ptr(out), n_entries, heads, groups, d, dv,
+                                           ctypes.c_float(unit_eps), _code(fresh.dtype), self._stream()), "delta_scan")
+        return out
+
+    # ---------------------------------------------------- sigmoid router with groups, ungated experts
+    def route_sigmoid(self, logits: torch.Tensor, correction: torch.Tensor, n_groups: int, keep_groups: int,
+                      chosen: torch.Tensor, weights: torch.Tensor) -> None:
+        """For every row of float32 `logits` [T, E]: s = sigmoid(logit); choice scores s + correction; with n_groups > 0 only
+        experts of the keep_groups best groups (a group is worth its two largest choice scores) can be chosen; the `top`
+        largest choice scores (chosen int32 [T, top], falling, the lower index of equals first), weighted by their s over
+        the chosen's sum + 1e-20 (weights float32 [T, top])."""
+        _dev(logits, correction, chosen, weights)
+        n_tokens, n_experts = logits.shape
+        top = chosen.shape[1]
+        _need(logits.dtype == torch.float32 and correction.dtype == torch.float32 and correction.numel() == n_experts,
+              "router logits and the correction are float32")
+        _need(chosen.dtype == torch.int32 and weights.dtype == torch.float32
+              and tuple(chosen.shape) == (n_tokens, top) == tuple(weights.shape), "chosen int32 and weights float32 [T, top]")
+        _need(0 < top <= min(n_experts, 64) and n_experts <= 1024, "between one and 64 of up to 1024 experts a token")
+        _need(n_groups == 0 or (n_experts % n_groups == 0 and 0 < keep_groups <= n_groups
+                                and keep_groups * (n_experts // n_groups) >= top), "the groups do not fit")
+        self._check(self.lib.ta_route_sigmoid(_ptr(logits), _ptr(correction), n_tokens, n_experts, int(n_groups), int(keep_groups),
+                                              top, _ptr(chosen), _ptr(weights), self._stream()), "route_sigmoid")
+
+    def expert_act(self, up: torch.Tensor, chosen: torch.Tensor, weights: torch.Tensor, n_experts: int, inner: int,
+                   out: torch.Tensor) -> torch.Tensor:
+        """up [T, n_experts inner] -> out [T, >= n_experts inner]: weight * max(up, 0)^2 in the columns of the experts a
+        token chose, zero everywhere else."""
+        _dev(up, chosen, weights, out)
+        n_tokens = up.shape[0]
+        _need(up.shape[1] == n_experts * inner, "up width")
+        _need(out.shape[0] == n_tokens and out.shape[1] >= n_experts * inner and out.dtype == up.dtype, "out is [T, >= E inner]")
+        _need(chosen.dtype == torch.int32 and weights.dtype == torch.float32 and chosen.shape == weights.shape
+              and chosen.shape[0] == n_tokens, "chosen and weights [T, top]")
+        self._check(self.lib.ta_expert_act(_ptr(up), _ptr(chosen), _ptr(weights), n_tokens, chosen.shape[1], n_experts, inner,
+                                           out.shape[1], _ptr(out), _code(out.dtype), self._stream()), "expert_act")
+        return out
+
+    def relu2(self, x: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+        """out = max(x, 0)^2, element by element."""
+        _dev(x, out)
+        _need(x.shape == out.shape and x.dtype == out.dtype, "relu2 shapes do not fit")
+        self._check(self.lib.ta_relu2(_ptr(x), _ptr(out), ctypes.c_size_t(x.numel()), _code(x.dtype), self._stream()), "relu2")
         return out
 
     def norm_add_rmsnorm(self, residual: torch.Tensor, delta: torch.Tensor | None, post_weight: torch.Tensor | None,

@@ -28,7 +28,9 @@ class RMSNorm(Norm):
 
     @staticmethod
     def tensor_specs(spec: NormSpec) -> dict[str, TensorSpec]:
-        return {spec.options.get("tensor_name", "weight"): TensorSpec((spec.size,), init="ones", role="vector")}
+        # (A weight that is stored around zero is drawn around zero.)
+        return {spec.options.get("tensor_name", "weight"): TensorSpec((spec.size,), role="vector",
+                                                                      init="near_zero" if spec.options.get("offset") else "ones")}
 
     def fold(self):
         return NormFold(self.weight, self.eps)

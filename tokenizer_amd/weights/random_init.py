@@ -42,6 +42,9 @@ def random_tensor(name: str, spec: TensorSpec, seed: int, norm_spread: float = 0
         return (torch.eye(spec.shape[0], spec.shape[1]) + float(norm_spread) * noise).to(torch.bfloat16)
     if spec.init == "zeros":
         return torch.zeros(spec.shape, dtype=torch.bfloat16)
+    if spec.init == "near_zero":           # a norm's scale stored as its distance from 1
+        noise = torch.empty(spec.shape, dtype=torch.float32).normal_(0.0, 1.0, generator=_generator(seed, name))
+        return (float(norm_spread) * noise).to(torch.bfloat16)
     if spec.init != "normal":
         raise ValueError(f"unknown init {spec.init!r} for {name}")
     values = torch.empty(spec.shape, dtype=torch.float32)
