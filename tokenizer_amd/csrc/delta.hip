@@ -43,7 +43,12 @@ short_conv_silu_kernel(const T* __restrict__ rows, int row_stride, ConvRuns runs
                        const int* __restrict__ state_slots, const int* __restrict__ entry_of_token, T* __restrict__ out) {
   const int t = blockIdx.x, c = blockIdx.y * 256 + threadIdx.x;
   if (c >= channels) return;
-  const int e = entry_of_token[t], lo = cu_q[e];
+  const int e = entry_of_token[t];
+  if (e < 0) {                                               // a token that only fills the batch up
+    st(out + (size_t)t * channels + c, 0.f);
+    return;
+  }
+  const int lo = cu_q[e];
   const bool zeros = first_position[e] == 0;
   const float* tail = state + (size_t)state_slots[e] * state_stride + state_offset;
   const int column = conv_column(runs, c);
