@@ -1,0 +1,634 @@
+"""Bokulorn through the framework against the plain implementation of tests/plain/bokulorn_plain.py.
+
+Every test runs on three backends: the engine on the CPU with the plain torch ops standing in for the kernel
+library (the host side: tables, slots, cache units, batching), and the engine on the GPU in float32 and in bfloat16
+(the HIP kernels).  The models are the tiny ones of bokulorn_configs.py with sharpened weights; the mechanisms alone
+run as the framework's own parts (the registered mixers and feed-forward) over a cache manager and pools of their own.
+"""
+import numpy as np
+import pytest
+import torch
+
+import trace_tools as tt
+from bokulorn_configs import BOKULORN, random_config, write_model
+from plain import bokulorn_plain as plain
+from tiny_configs import random_ids
+
+BACKENDS = [pytest.param("cpu", id="cpu"),
+            pytest.param("gpu-float32", marks=pytest.mark.gpu, id="gpu-float32"),
+            pytest.param("gpu-bfloat16", marks=pytest.mark.gpu, id="gpu-bfloat16")]
+# float32: sums in another order, against logits of order 1.  bfloat16 rounds the activations between the kernels and
+# the sharpened weights carry that further than a trained model's would: there the bound is on each row's root mean
+# square error against the row's own spread (a lost key, a state that starts from zeros in the middle of a sequence or
+# a convolution that forgets its last inputs moves a row by its whole spread; float32 pins the same kernels' indexing
+# to five digits).
+TOL = {"cpu": 2e-5, "gpu-float32": 1e-4, "gpu-bfloat16": 0.15}
+
+
+@pytest.fixture(scope="module")
+def folders(tmp_path_factory):
+    root = tmp_path_factory.mktemp("bokulorn")
+    return {name: write_model(raw, seed, str(root / name)) for name, (raw, seed) in BOKULORN.items()}
+
+
+@pytest.fixture(scope="module")
+def oracle(folders):
+    cache = {}
+
+    def get(name, ids):
+        key = (name, tuple(ids))
+        if key not in cache:
+            cfg, tensors = plain.load_folder(folders[name])
+            cache[key] = plain.forward(cfg, tensors, list(ids)).to(torch.float32)
+        return cache[key]
+    return get
+
+
+def make_engine(folder, backend, **kw):
+    from tokenizer_amd.engine import Engine, load_model
+    if backend == "cpu":
+        from kernel_refs import PlainOps
+        return Engine(load_model(folder, "float32", "cpu", ops=PlainOps()), **kw)
+    return Engine(load_model(folder, backend.split("-")[1]), **kw)
+
+
+def close(got, want, backend, what=""):
+    got = got.float().cpu()
+    if backend == "gpu-bfloat16":
+        spread = (want - want.mean(dim=-1, keepdim=True)).pow(2).mean(dim=-1).sqrt()
+        off = (got - want).pow(2).mean(dim=-1).sqrt() / spread
+        # (A router's choice scores for two experts are now and then nearly equal; bfloat16 rounding then picks the
+        # other expert, and that row, and the rows behind it that read it through the state or the cache, move by a
+        # good part of their spread.  Such rows are few.)
+        assert int((off > TOL[backend]).sum()) <= max(2, off.numel() // 10) and float(off.median()) <= TOL[backend] / 2, \
+            f"{what}: rows are off by up to {float(off.max())} of their spread, {int((off > TOL[backend]).sum())} over the bound"
+        return
+    err = float((got - want).abs().max())
+    bound = TOL[backend] * max(float(want.abs().max()), 1.0)
+    assert err <= bound, f"{what}: max abs error {err} against a bound of {bound}"
+
+
+def requests_for(name, lengths=(1, 2, 3, 21, 50, 97, 64, 33)):
+    vocab = BOKULORN[name][0]["vocab"]
+    return {f"r{i}": random_ids(vocab, n, 40 + i) for i, n in enumerate(lengths)}
+
+
+def check_trace(folders, oracle, name, backend, steps, reqs, **kw):
+    eng = make_engine(folders[name], backend, max_tokens=tt.peak_tokens(steps), max_requests=4, **kw)
+    eng.pools.poison()          # pages and state rows that no request wrote read as NaN
+    got = tt.run_in_process(eng, steps)
+    for rid, ids in reqs.items():
+        close(got[rid], oracle(name, ids), backend, rid)
+    eng.cache.check_invariants()
+    assert not eng.cache.requests
+    return eng
+
+
+NAMES = list(BOKULORN)
+
+
+# ------------------------------------------------------------------ whole models through the engine
+@pytest.mark.parametrize("backend", BACKENDS)
+@pytest.mark.parametrize("name", NAMES)
+def test_whole_prompts_and_the_first_tokens(folders, oracle, name, backend):
+    reqs = requests_for(name)
+    check_trace(folders, oracle, name, backend, tt.whole(reqs), reqs)
+
+
+@pytest.mark.parametrize("backend", BACKENDS)
+@pytest.mark.parametrize("name", NAMES)
+def test_prefill_then_token_by_token(folders, oracle, name, backend):
+    # The tail of 50 passes page borders of 16 and carries state and the convolutions' inputs from a prompt into
+    # single tokens; a request of 51 starts decoding behind its very first token.
+    reqs = requests_for(name, (60, 97, 64, 51))
+    check_trace(folders, oracle, name, backend, tt.decode_tail(reqs, 50), reqs)
+
+
+@pytest.mark.parametrize("backend", BACKENDS)
+@pytest.mark.parametrize("name", NAMES)
+@pytest.mark.parametrize("seed", [3, 4])
+def test_portions_down_to_two_tokens(folders, oracle, name, backend, seed):
+    reqs = requests_for(name, (97, 50, 64, 7))
+    steps = tt.portions(reqs, seed)
+    assert any(len(s["entries"][0]["tokens"]) == 2 for s in steps)
+    check_trace(folders, oracle, name, backend, steps, reqs)
+
+
+@pytest.mark.parametrize("backend", BACKENDS)
+@pytest.mark.parametrize("name", NAMES)
+@pytest.mark.parametrize("seed", [6, 7])
+def test_mixed_batches_with_pages_and_slots_used_again(folders, oracle, name, backend, seed):
+    reqs = requests_for(name, (33, 97, 21, 64, 50, 80, 12, 45, 3, 70))
+    steps = tt.mixed(reqs, seed, max_live=4, tail=14)
+    assert max(len(s["entries"]) for s in steps) >= 3
+    eng = check_trace(folders, oracle, name, backend, steps, reqs)
+    assert eng.cache.max_requests == 4          # ten requests went through four slots
+
+
+@pytest.mark.parametrize("backend", BACKENDS)
+@pytest.mark.parametrize("page_size", [16, 48])
+def test_other_page_sizes_and_batches_against_each_request_alone(folders, oracle, backend, page_size):
+    from tokenizer_amd.engine import StepEntry
+    name = "A"
+    reqs = requests_for(name, (70, 9, 31))
+    eng = make_engine(folders[name], backend, num_pages=24, page_size=page_size, max_requests=3)
+    eng.pools.poison()
+    for rid in reqs:
+        eng.add_request(rid)
+    heads = {rid: len(ids) - 5 for rid, ids in reqs.items()}
+    got = {rid: [] for rid in reqs}
+    logits = eng.step([StepEntry(rid, ids[:heads[rid]], list(range(heads[rid]))) for rid, ids in reqs.items()]).float().cpu()
+    row = 0
+    for rid in reqs:
+        got[rid].append(logits[row:row + heads[rid]])
+        row += heads[rid]
+    for k in range(5):
+        logits = eng.step([StepEntry(rid, [ids[heads[rid] + k]], [0]) for rid, ids in reqs.items()]).float().cpu()
+        for row, rid in enumerate(reqs):
+            got[rid].append(logits[row:row + 1])
+    for rid, ids in reqs.items():
+        close(torch.cat(got[rid]), oracle(name, ids), backend, rid)
+
+
+@pytest.mark.parametrize("backend", BACKENDS)
+@pytest.mark.parametrize("name", ["A", "C"])
+def test_long_decoding(folders, oracle, name, backend):
+    ids = random_ids(BOKULORN[name][0]["vocab"], 230, 77)
+    reqs = {"long": ids}
+    check_trace(folders, oracle, name, backend, tt.decode_tail(reqs, tail=227), reqs)
+
+
+@pytest.mark.parametrize("backend", BACKENDS)
+def test_greedy_generation_through_the_entry_point_and_the_scheduler(folders, backend):
+    from tokenizer_amd.engine import GenerateParams, Scheduler, SchedulerConfig, generate
+    name = "A"
+    cfg, tensors = plain.load_folder(folders[name])
+    prompts = [random_ids(cfg["vocab"], n, 90 + n) for n in (11, 30, 4)]
+    want = [plain.greedy_generate(cfg, tensors, p, 9) for p in prompts]
+    eng = make_engine(folders[name], backend, num_pages=16, max_requests=4)
+    eng.pools.poison()
+    alone = [generate(eng, p, GenerateParams.greedy(9)).tokens for p in prompts]
+    sched = Scheduler(eng, SchedulerConfig(num_blocks=16, max_batch_size=4))
+    rids = [sched.add_request(p, GenerateParams.greedy(9)) for p in prompts]
+    results = sched.run()
+    together = [results[rid].tokens for rid in rids]
+    assert alone == together
+    if backend != "gpu-bfloat16":           # (bfloat16 may pick another of two near-equal logits)
+        assert alone == want
+    else:
+        for prompt, picked in zip(prompts, alone):
+            logits = plain.forward(cfg, tensors, prompt + picked)[len(prompt) - 1:-1]
+            for row, token in zip(logits, picked):
+                assert float(row.max() - row[token]) <= 0.2 * float(row.std())
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("cut", ["whole", "tail", "portions", "mixed"])
+def test_hundreds_of_tokens(folders, oracle, dtype, cut):
+    """Prompts long enough for the prompt kernels' tiles, the sorted routed layers and the scan's groups of tokens."""
+    name = "C"
+    reqs = requests_for(name, (300, 17, 411, 130))
+    steps = {"whole": lambda: tt.whole(reqs), "tail": lambda: tt.decode_tail(reqs, 40),
+             "portions": lambda: tt.portions(reqs, 11), "mixed": lambda: tt.mixed(reqs, 12, max_live=4, tail=10)}[cut]()
+    check_trace(folders, oracle, name, f"gpu-{dtype}", steps, reqs)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_the_replay_program_on_a_model_folder(folders, oracle, tmp_path, dtype):
+    name = "B"
+    reqs = requests_for(name, (40, 23, 5, 64, 31))
+    steps = tt.mixed(reqs, 9, max_live=4, tail=6)
+    got = tt.run_program(folders[name], dtype, steps, str(tmp_path / "out"), tt.peak_tokens(steps), BOKULORN[name][0]["vocab"])
+    for rid, ids in reqs.items():
+        close(got[rid], oracle(name, ids), f"gpu-{dtype}", rid)
+
+
+@pytest.mark.parametrize("backend", BACKENDS)
+@pytest.mark.parametrize("seed", list(range(1, 17)))
+def test_models_drawn_from_a_seed(tmp_path, backend, seed):
+    """Other numbers and orders of layers, sizes and constants; whole, then cut and batched."""
+    raw = random_config(seed)
+    folder = write_model(raw, 100 + seed, str(tmp_path / "m"), sharpen=3.0)
+    cfg, tensors = plain.load_folder(folder)
+    reqs = {f"r{i}": random_ids(raw["vocab"], n, seed * 10 + i) for i, n in enumerate((37, 5, 52))}
+    steps = tt.mixed(reqs, seed, max_live=3, tail=5) if seed % 2 else tt.portions(reqs, seed)
+    eng = make_engine(folder, backend, max_tokens=tt.peak_tokens(steps), max_requests=3)
+    eng.pools.poison()
+    got = tt.run_in_process(eng, steps)
+    for rid, ids in reqs.items():
+        close(got[rid], plain.forward(cfg, tensors, ids).float(), backend, f"seed {seed} {rid}")
+
+
+# ------------------------------------------------------------------ configuration, registry, schedule
+def test_a_layer_with_another_layers_tensors_has_a_cache_unit_of_its_own():
+    from tokenizer_amd.config import BokulornConfig
+    from tokenizer_amd.models.bokulorn import bokulorn_spec
+    from tokenizer_amd.parts import cache_needs, expected_tensors
+    raw = BOKULORN["B"][0]
+    cfg = BokulornConfig.from_dict(raw)
+    spec = bokulorn_spec(cfg)
+    assert len(spec.layers) == 3 and len(spec.schedule) == 5
+    assert [entry.layer for entry in spec.schedule] == [0, 1, 2, 1, 1]        # layer 4 names 3, which names 1
+    units = [entry.cache_unit() for entry in spec.schedule]
+    assert len(set(units)) == 5                                                   # state and cache are never shared
+    needs = cache_needs(spec)
+    assert len(needs) == 5 and needs[3].state_shape == needs[1].state_shape and needs[3].state_shape is not None
+    names = set(expected_tensors(spec))
+    assert "l1.mix.q.conv" in names and "l0.mix.dkv.norm" in names and not any(n.startswith(("l3.", "l4.")) for n in names)
+
+
+def test_a_config_with_a_missing_or_misfitting_key_is_refused():
+    import copy
+    from tokenizer_amd.config import BokulornConfig, ConfigError
+    raw = BOKULORN["A"][0]
+    BokulornConfig.from_dict(raw)
+
+    def broken(change):
+        bad = copy.deepcopy(raw)
+        change(bad)
+        with pytest.raises(ConfigError):
+            BokulornConfig.from_dict(bad)
+    broken(lambda c: c["layers"][0]["mixer"].pop("conv"))
+    broken(lambda c: c["layers"][0]["mixer"].update(kv_heads=3))
+    broken(lambda c: c["layers"][1]["mixer"].pop("kv_rank"))
+    broken(lambda c: c["layers"][1]["mixer"]["rot"].update(dims=6))
+    broken(lambda c: c["layers"][2].update(type="attention"))
+    broken(lambda c: c["layers"][0]["mlp"]["router"]["groups"].update(keep=4))
+    broken(lambda c: c["layers"][0]["mlp"]["router"].update(top=5))           # two kept groups of two hold four
+    broken(lambda c: c["layers"][3].update(weights_of=3))
+    broken(lambda c: c["layers"][3].update(weights_of=9))
+    broken(lambda c: c["norm"].pop("eps"))
+
+
+def test_the_command_line_knows_the_design(folders):
+    from tokenizer_amd.config import load_config
+    cfg = load_config(folders["D"])
+    assert cfg.architecture == "Bokulorn" and cfg.embedding_scale == 1.0 and len(cfg.layers) == 2
+
+
+# ------------------------------------------------------------------ mechanisms alone
+def ops_for(backend):
+    if backend == "cpu":
+        from kernel_refs import PlainOps
+        return PlainOps(), torch.device("cpu"), torch.float32
+    from tokenizer_amd.kernels import get_ops
+    return get_ops(), torch.device("cuda:0"), (torch.float32 if backend.endswith("float32") else torch.bfloat16)
+
+
+def rounded(x, dtype):
+    """Random float64 data as the compute dtype holds it."""
+    return x.to(dtype).to(torch.float64)
+
+
+def tolerance(dtype, exact=2e-5, rough=3e-2):
+    return rough if dtype == torch.bfloat16 else exact
+
+
+class PartRunner:
+    """One mixer of the framework over a cache manager and pools of its own: requests are fed in steps of
+    (request, rows) and give their outputs back in order.  Pages and state rows start as NaN."""
+
+    def __init__(self, kind, spec, tensors, backend, num_pages=40, page_size=16, max_requests=3):
+        from tokenizer_amd.cache import CacheManager, CachePools
+        from tokenizer_amd.parts import MIXERS, LayerCache, Runtime
+        self.ops, self.device, self.dtype = ops_for(backend)
+        cls = MIXERS.get(kind)
+        need = cls.cache_need(spec)
+        self.manager = CacheManager([need], num_pages=num_pages, page_size=page_size, max_requests=max_requests)
+        self.pools = CachePools(self.manager, [need], self.dtype, self.device)
+        self.pools.poison()
+        stored = {}
+        for name, t in tensors.items():
+            vector = t.dim() == 1 or name.endswith(".conv")
+            stored[name] = t.to(torch.float32 if vector else self.dtype).to(self.device).contiguous()
+        self.part = cls(spec, stored, Runtime(self.dtype, self.device, self.ops))
+        k_pages, v_pages = self.pools.layer_pages(0)
+        self.cache = LayerCache(group=self.manager.group_of_layer[0], k_pages=k_pages, v_pages=v_pages,
+                                state=self.pools.states.get(0))
+
+    def step(self, parts):
+        """parts: [(request id, rows [n, width] float64)] -> their outputs, float64 on the CPU."""
+        from tokenizer_amd.engine.batch import StepEntry, build_context
+        entries = []
+        for rid, rows in parts:
+            if not self.manager.has_request(rid):
+                self.manager.add_request(rid)
+            assert self.manager.reserve(rid, self.manager.seq_len(rid) + rows.shape[0])
+            entries.append(StepEntry(rid, [0] * rows.shape[0], []))
+        ctx = build_context(entries, self.manager, self.device)
+        x = torch.cat([rows for _, rows in parts]).to(self.dtype).to(self.device).contiguous()
+        out = self.part.forward(x, ctx, self.cache).double().cpu()
+        got, row = [], 0
+        for rid, rows in parts:
+            got.append(out[row:row + rows.shape[0]])
+            row += rows.shape[0]
+            self.manager.advance(rid, self.manager.seq_len(rid) + rows.shape[0])
+        return got
+
+    def run(self, h, cuts, rid="main", rider=None):
+        """The sequence h [n, width] in steps of `cuts` rows; `rider`: rows of another request that go along, one a step."""
+        out, at = [], 0
+        for number, size in enumerate(cuts):
+            parts = [(rid, h[at:at + size])]
+            if rider is not None and number < rider.shape[0]:
+                parts.insert(number % 2, ("rider", rider[number:number + 1]))
+            got = self.step(parts)
+            out.append(got[[p[0] for p in parts].index(rid)])
+            at += size
+        assert at == h.shape[0]
+        return torch.cat(out)
+
+    def end(self, rid):
+        self.manager.release(rid)
+
+
+CUTS = {"prompt": lambda n: [n], "portions": lambda n: [37, 2, 16, 1, 1, 29] + [n - 86],
+        "decoded": lambda n: [n - 70] + [1] * 70}
+
+
+def latent_spec(rotated, width, heads, d, dv, q_rank, kv_rank, rot_dim, scale, base, eps):
+    from tokenizer_amd.parts import MixerSpec
+    return MixerSpec("latent_attention", hidden_size=width, n_heads=heads, n_kv_heads=1, head_dim=d, value_dim=dv,
+                     scale=scale, q_rank=q_rank, kv_rank=kv_rank, rot_dim=rot_dim if rotated else 0, head_gate=rotated,
+                     element_gate=not rotated, eps=eps, options={"rot_base": base})
+
+
+def latent_tensors(gen, rotated, width, heads, d, dv, q_rank, kv_rank, rot_dim, dtype, size=1.0):
+    e = rot_dim if rotated else 0
+    rand = lambda *shape: torch.randn(*shape, generator=gen, dtype=torch.float64)
+    w = {"dq": rand(q_rank, width) * size / width ** 0.5, "dq.norm": 1 + 0.3 * rand(q_rank),
+         "uq": rand(heads * (d + e), q_rank) * size / q_rank ** 0.5,
+         "dkv": rand(kv_rank + e, width) * size / width ** 0.5, "dkv.norm": 1 + 0.3 * rand(kv_rank),
+         "uk": rand(heads * d, kv_rank) * size / kv_rank ** 0.5, "uv": rand(heads * dv, kv_rank) / kv_rank ** 0.5,
+         "g": rand(heads if rotated else heads * dv, width) / width ** 0.5, "o": rand(width, heads * dv) / (heads * dv) ** 0.5}
+    return {name: (t.float().double() if t.dim() == 1 else rounded(t, dtype)) for name, t in w.items()}
+
+
+@pytest.mark.parametrize("backend", BACKENDS)
+@pytest.mark.parametrize("cut", list(CUTS))
+@pytest.mark.parametrize("rotated,width,heads,d,dv,q_rank,kv_rank,rot_dim,scale,base", [
+    (True, 48, 4, 16, 24, 24, 40, 8, 0.3, 10000.0), (True, 40, 3, 10, 14, 20, 22, 6, 0.35, 300.0),
+    (True, 32, 1, 24, 40, 16, 30, 2, 0.2, 100.0), (True, 64, 2, 32, 32, 48, 112, 16, 0.18, 500000.0),
+    (False, 48, 2, 32, 16, 32, 32, 0, 0.2, 1.0), (False, 40, 3, 6, 10, 12, 18, 0, 0.4, 1.0),
+    (False, 64, 4, 16, 64, 64, 96, 0, 0.25, 1.0)])
+def test_latent_attention_alone(backend, cut, rotated, width, heads, d, dv, q_rank, kv_rank, rot_dim, scale, base):
+    ops, device, dtype = ops_for(backend)
+    gen = torch.Generator().manual_seed(heads * 100 + d + kv_rank)
+    n, eps = 120, 1e-5
+    w = latent_tensors(gen, rotated, width, heads, d, dv, q_rank, kv_rank, rot_dim, dtype, size=3.0)
+    h = rounded(torch.randn(n, width, generator=gen, dtype=torch.float64), dtype)
+    m = {"heads": heads, "dim": d, "vdim": dv, "kv_rank": kv_rank, "rot_dim": rot_dim, "scale": scale,
+         "rot": {"base": base, "dims": rot_dim}}
+    want = plain.latent_attention(h, m, w, eps, rotated)
+    runner = PartRunner("latent_attention", latent_spec(rotated, width, heads, d, dv, q_rank, kv_rank, rot_dim, scale, base, eps),
+                        w, backend)
+    got = runner.run(h, CUTS[cut](n), rider=h[:9] * 0.5)
+    assert float((got - want).abs().max()) <= tolerance(dtype, 3e-5, 5e-2) * max(1.0, float(want.abs().max()))
+    if rotated:         # the positions do matter: the same rows with every position one further give other outputs
+        shifted = plain.latent_attention(torch.cat([h[:1], h]), m, w, eps, True)[1:]
+        assert float((shifted - want).abs().max()) > 0.05
+
+
+@pytest.mark.parametrize("backend", BACKENDS)
+@pytest.mark.parametrize("cut", list(CUTS))
+@pytest.mark.parametrize("rotated", [True, False])
+def test_one_key_made_to_stand_out_far_back_and_at_page_borders(backend, cut, rotated):
+    """The mixer's input is [a query part | a key part]: the query latent reads the first half, the key latent the
+    second, and both go up through the same matrix, so a query whose first half is the second half of a chosen
+    token scores that token far above all others.  The chosen keys are, in turn: the second token of the sequence
+    (hundreds of tokens back), the keys on either side of the last page border, the key before the query, and the
+    query itself.  A key that is lost, or one too many, changes the output by all of it."""
+    ops, device, dtype = ops_for(backend)
+    half, heads, dv, n, eps = 16, 2, 8, 230, 1e-6
+    rot_dim = 4 if rotated else 0
+    gen = torch.Generator().manual_seed(5 + rotated)
+    rand = lambda *shape: torch.randn(*shape, generator=gen, dtype=torch.float64)
+    keys = rand(n, half)
+    keys = keys / keys.norm(dim=-1, keepdim=True)
+    target = []
+    for i in range(n):
+        j = [1, i - i % 16, i - i % 16 - 1, i - 1, i, 0][i % 6]
+        target.append(j if 0 <= j <= i else i)
+    h = rounded(torch.cat([keys[target], keys], dim=1), dtype)
+    up = torch.linalg.qr(rand(half, half))[0]
+    eye = torch.eye(half, dtype=torch.float64)
+    zero = torch.zeros(half, half, dtype=torch.float64)
+    w = {"dq": torch.cat([eye, zero], dim=1), "dq.norm": torch.ones(half, dtype=torch.float64),
+         "uq": torch.cat([torch.cat([up, 0.02 * rand(rot_dim, half)]) for _ in range(heads)]),
+         "dkv": torch.cat([torch.cat([zero, eye], dim=1), 0.3 * rand(rot_dim, 2 * half)]),
+         "dkv.norm": torch.ones(half, dtype=torch.float64), "uk": torch.cat([up] * heads),
+         "uv": rand(heads * dv, half), "g": 0.1 * rand(heads if rotated else heads * dv, 2 * half),
+         "o": torch.eye(heads * dv, dtype=torch.float64)[:2 * half].t().contiguous() if heads * dv >= 2 * half
+         else torch.cat([torch.eye(heads * dv, dtype=torch.float64), torch.zeros(2 * half - heads * dv, heads * dv, dtype=torch.float64)])}
+    w = {name: (t if t.dim() == 1 else rounded(t, dtype)) for name, t in w.items()}
+    scale = 1.5                 # the latents have unit RMS: a matching pair scores 16 * 1.5, others around +-6
+    m = {"heads": heads, "dim": half, "vdim": dv, "kv_rank": half, "rot_dim": rot_dim, "scale": scale,
+         "rot": {"base": 100.0, "dims": rot_dim}}
+    want = plain.latent_attention(h, m, w, eps, rotated)
+    runner = PartRunner("latent_attention", latent_spec(rotated, 2 * half, heads, half, dv, half, half, rot_dim, scale, 100.0, eps),
+                        w, backend)
+    got = runner.run(h, CUTS[cut](n), rider=h[:7])
+    assert float((got - want).abs().max()) <= tolerance(dtype, 3e-5, 5e-2) * float(want.abs().max())
+    # The chosen keys do carry the outputs: without the second token, rows that chose it move by far more.
+    blind = h.clone()
+    blind[1, half:] = -blind[1, half:]
+    moved = plain.latent_attention(blind, m, w, eps, rotated)
+    rows = [i for i in range(40, n) if target[i] == 1]
+    assert len(rows) > 20 and float((moved[rows] - want[rows]).abs().max(dim=-1).values.min()) > 0.2
+
+
+def delta_spec(width, heads, groups, d, dv, taps, eps, low):
+    from tokenizer_amd.parts import MixerSpec
+    return MixerSpec("gated_delta", hidden_size=width, n_heads=heads, n_kv_heads=groups, head_dim=d, value_dim=dv,
+                     conv_taps=taps, eps=eps, options={"unit_eps": 1e-6, "low_rank": low})
+
+
+def delta_tensors(gen, width, heads, groups, d, dv, taps, low, dtype, size=2.0):
+    rand = lambda *shape: torch.randn(*shape, generator=gen, dtype=torch.float64)
+    w = {"q": rand(groups * d, width) * size / width ** 0.5, "k": rand(groups * d, width) * size / width ** 0.5,
+         "v": rand(heads * dv, width) * size / width ** 0.5, "b": rand(heads, width) * size / width ** 0.5,
+         "q.conv": rand(groups * d, taps) * 0.6, "k.conv": rand(groups * d, taps) * 0.6, "v.conv": rand(heads * dv, taps) * 0.6,
+         "a1": rand(low, width) / width ** 0.5, "a2": rand(heads * d, low) * 2.0, "dt_bias": rand(heads * d) - 1.0,
+         "A_log": rand(heads) * 0.5 - 0.5, "g1": rand(low, width) / width ** 0.5, "g2": rand(heads * dv, low) * 2.0,
+         "norm": 1 + 0.3 * rand(dv), "o": rand(width, heads * dv) / (heads * dv) ** 0.5}
+    return {name: (t.float().double() if t.dim() == 1 or name.endswith(".conv") else rounded(t, dtype)) for name, t in w.items()}
+
+
+def delta_bound(dtype):
+    # (bfloat16: q, k and v pass the convolution and its activation in bfloat16, and the head norm brings every
+    # output to unit size whatever its scale was, so a rounding of 2^-9 is carried by a handful of steps.)
+    return tolerance(dtype, 5e-5, 8e-2)
+
+
+@pytest.mark.parametrize("backend", BACKENDS)
+@pytest.mark.parametrize("cut", list(CUTS))
+@pytest.mark.parametrize("width,heads,groups,d,dv,taps,low", [(48, 4, 2, 16, 24, 4, 8), (40, 3, 3, 12, 14, 2, 5), (32, 2, 1, 20, 8, 1, 16),
+                                                            (64, 4, 1, 64, 32, 5, 24), (32, 2, 2, 128, 40, 3, 8), (24, 1, 1, 8, 72, 6, 3)])
+def test_the_delta_rule_alone_with_its_state_in_a_slot(backend, cut, width, heads, groups, d, dv, taps, low):
+    ops, device, dtype = ops_for(backend)
+    gen = torch.Generator().manual_seed(heads * 1000 + d * 10 + taps)
+    n, eps = 120, 1e-5
+    w = delta_tensors(gen, width, heads, groups, d, dv, taps, low, dtype)
+    h = rounded(torch.randn(n, width, generator=gen, dtype=torch.float64), dtype)
+    m = {"heads": heads, "kv_heads": groups, "dim": d, "vdim": dv, "conv": taps}
+    want = plain.channel_delta(h, m, w, eps)
+    runner = PartRunner("gated_delta", delta_spec(width, heads, groups, d, dv, taps, eps, low), w, backend, max_requests=2)
+    got = runner.run(h, CUTS[cut](n), rider=h[50:59])
+    assert float((got - want).abs().max()) <= delta_bound(dtype) * max(1.0, float(want.abs().max()))
+    # The slot is given back and taken again: the next request starts from zeros, not from what the slot holds.
+    runner.end("main")
+    runner.end("rider")
+    again = runner.run(h[:30], [4, 1, 25], rid="next")
+    assert float((again - want[:30]).abs().max()) <= delta_bound(dtype) * max(1.0, float(want.abs().max()))
+
+
+@pytest.mark.parametrize("backend", BACKENDS)
+@pytest.mark.parametrize("cut", list(CUTS))
+def test_a_write_far_back_is_read_through_the_state(backend, cut):
+    """Decays of nearly one (a large negative bias in front of the softplus) and step sizes of nearly one.  The second
+    token writes under a key coordinate that no later token writes to (the rule overwrites what later keys overlap with,
+    so only such a write stays), and two hundred tokens later the rows whose query is that coordinate read its value
+    back.  A state that is lost at the edge of a portion shows in all of them."""
+    ops, device, dtype = ops_for(backend)
+    width, heads, groups, d, dv, taps, low, n, eps = 32, 2, 1, 16, 16, 1, 4, 230, 1e-6
+    gen = torch.Generator().manual_seed(12)
+    rand = lambda *shape: torch.randn(*shape, generator=gen, dtype=torch.float64)
+    w = delta_tensors(gen, width, heads, groups, d, dv, taps, low, dtype)
+    eye, zero = torch.eye(d, dtype=torch.float64), torch.zeros(d, d, dtype=torch.float64)
+    w["q"], w["k"] = torch.cat([eye, zero], dim=1) * 4, torch.cat([zero, eye], dim=1) * 4     # silu(4 x) keeps the direction's positive part
+    w["q.conv"], w["k.conv"] = torch.ones(d, 1, dtype=torch.float64), torch.ones(d, 1, dtype=torch.float64)
+    w["a2"] = torch.zeros_like(w["a2"])
+    w["dt_bias"] = torch.full_like(w["dt_bias"], -9.0)
+    w["b"] = torch.zeros_like(w["b"])
+    w["b"][:, 0] = 3.0
+    keys = rand(n, d).abs()
+    keys[:, :2] = 0
+    keys[1] = 0
+    keys[1, 1] = 1.0                                            # the second token's key: a coordinate of its own
+    keys = keys / keys.norm(dim=-1, keepdim=True)
+    target = [[1, i - 1, i, 1][i % 4] if i > 1 else i for i in range(n)]
+    h = torch.cat([keys[target], keys], dim=1)
+    h[:, 0] = 2.0                                               # beta = sigmoid(6): the whole step
+    h = rounded(h, dtype)
+    m = {"heads": heads, "kv_heads": groups, "dim": d, "vdim": dv, "conv": taps}
+    want = plain.channel_delta(h, m, w, eps)
+    runner = PartRunner("gated_delta", delta_spec(width, heads, groups, d, dv, taps, eps, low), w, backend, max_requests=2)
+    got = runner.run(h, CUTS[cut](n), rider=h[3:12])
+    assert float((got - want).abs().max()) <= delta_bound(dtype) * max(1.0, float(want.abs().max()))
+    other = h.clone()
+    other[1, d:] = other[2, d:]                                # the second token writes under another key
+    moved = plain.channel_delta(other, m, w, eps)
+    rows = [i for i in range(150, n) if target[i] == 1]
+    assert len(rows) > 15 and float((moved[rows] - want[rows]).abs().max(dim=-1).values.min()) > 0.1
+
+
+@pytest.mark.parametrize("backend", BACKENDS)
+@pytest.mark.parametrize("taps", [1, 2, 4, 7])
+def test_the_short_convolution_keeps_its_last_inputs_across_steps(backend, taps):
+    """Only the oldest tap is set: the output at t is silu(x[t - taps + 1]), zeros before the start.  Steps of one
+    and two rows, shorter than the taps, pass inputs on that are older than the step before."""
+    ops, device, dtype = ops_for(backend)
+    gen = torch.Generator().manual_seed(taps)
+    widths, offsets, n = (10, 6, 20), (0, 16, 24), 41
+    channels = sum(widths)
+    x = rounded(torch.randn(n, 48, generator=gen, dtype=torch.float64), dtype)
+    weights = torch.zeros(channels, taps, dtype=torch.float64)
+    weights[:, 0] = 1.0
+    weights[::3, taps - 1] += 0.5
+    picked = torch.cat([x[:, o:o + k] for o, k in zip(offsets, widths)], dim=1)
+    want = plain.silu(plain.short_convolution(picked, weights))
+    state = torch.full((3, 7 + (taps - 1) * channels + 2), float("nan"), device=device)
+    got, at = [], 0
+    i32 = lambda values: torch.tensor(values, dtype=torch.int32, device=device)
+    for size in (1, 2, 1, 1, 9, 2, 2, 1, 17, 5):
+        rows = x[at:at + size].to(dtype).to(device).contiguous()
+        out = torch.empty((size, channels), dtype=dtype, device=device)
+        ops.short_conv_silu(rows, offsets, widths, weights.float().to(device), state, 7, i32([0, size]), i32([at]), i32([2]),
+                            i32([0] * size), out)
+        got.append(out.double().cpu())
+        at += size
+    assert at == n
+    assert float((torch.cat(got) - want).abs().max()) <= tolerance(dtype, 1e-6, 2e-2) * max(1.0, float(want.abs().max()))
+
+
+@pytest.mark.parametrize("backend", BACKENDS)
+@pytest.mark.parametrize("experts,top,count,keep", [(6, 2, 3, 2), (5, 1, 5, 5), (8, 3, 2, 1), (12, 4, 3, 2), (4, 2, 1, 1), (9, 3, 3, 1),
+                                                    (64, 6, 8, 3), (3, 3, 3, 3)])
+def test_the_sigmoid_router_with_groups(backend, experts, top, count, keep):
+    """Choice scores with the correction, weights without; groups worth their two best; what is outside the kept
+    groups counts as minus infinity also where choice scores are negative (corrections far below zero)."""
+    ops, device, dtype = ops_for(backend)
+    gen = torch.Generator().manual_seed(experts * 10 + top)
+    n = 200
+    logits = (torch.randn(n, experts, generator=gen, dtype=torch.float64) * 2).float()
+    for shift in (0.0, -3.0):
+        correction = (torch.randn(experts, generator=gen, dtype=torch.float64) * 0.4 + shift).float()
+        chosen = torch.empty((n, top), dtype=torch.int32, device=device)
+        weights = torch.empty((n, top), dtype=torch.float32, device=device)
+        ops.route_sigmoid(logits.to(device), correction.to(device), count, keep, chosen, weights)
+        s = torch.sigmoid(logits.double())
+        choice = s + correction.double()
+        per = experts // count
+        worth = torch.topk(choice.reshape(n, count, per), min(2, per), dim=-1).values.sum(-1)
+        for t in range(n):
+            groups = sorted(range(count), key=lambda g: -float(worth[t, g]))[:keep]
+            allowed = [e for e in range(experts) if e // per in groups]
+            best = sorted(allowed, key=lambda e: -float(choice[t, e]))[:top]
+            got = chosen[t].tolist()
+            assert sorted(got) == sorted(best), (t, got, best)
+            total = sum(float(s[t, e]) for e in got) + 1e-20
+            for e, a in zip(got, weights[t].tolist()):
+                assert abs(a - float(s[t, e]) / total) < 1e-5
+        assert shift == 0.0 or bool((choice < 0).all())
+
+@pytest.mark.parametrize("backend", BACKENDS)
+@pytest.mark.parametrize("experts,top,count,keep,inner,width,tokens", [(6, 2, 3, 2, 24, 64, 37), (5, 1, 5, 5, 10, 52, 9), (8, 3, 2, 1, 32, 128, 50),
+                                                                     (12, 4, 3, 2, 24, 40, 3), (8, 2, 4, 2, 32, 64, 700)])
+def test_the_routed_experts_without_a_gate_branch(backend, experts, top, count, keep, inner, width, tokens):
+    """The framework's routed feed-forward with the sigmoid router and squared-ReLU experts; 700 tokens take the
+    sorted form where the backend has one."""
+    from tokenizer_amd.parts import FEED_FORWARDS, FeedForwardSpec, Runtime
+    ops, device, dtype = ops_for(backend)
+    gen = torch.Generator().manual_seed(experts + inner)
+    rand = lambda *shape: torch.randn(*shape, generator=gen, dtype=torch.float64)
+    w = {"router": rounded(rand(experts, width) * 6 / width ** 0.5, dtype), "correction": (rand(experts) * 0.3).float().double()}
+    for e in range(experts):
+        w[f"e{e}.up"] = rounded(rand(inner, width) / width ** 0.5, dtype)
+        w[f"e{e}.down"] = rounded(rand(width, inner) / inner ** 0.5, dtype)
+    h = rounded(rand(tokens, width), dtype)
+    mlp = {"router": {"experts": experts, "top": top, "groups": {"count": count, "keep": keep}}}
+    want = plain.routed_feed_forward(h, mlp, w)
+    spec = FeedForwardSpec("routed_experts", hidden_size=width, intermediate_size=inner, activation="relu2", gated=False,
+                           n_experts=experts, top_k=top, router="sigmoid", n_groups=count, keep_groups=keep)
+    stored = {name: t.to(torch.float32 if t.dim() == 1 else dtype).to(device) for name, t in w.items()}
+    part = FEED_FORWARDS.get("routed_experts")(spec, stored, Runtime(dtype, device, ops))
+    got = part.forward(h.to(dtype).to(device), None).double().cpu()
+    err = (got - want).abs().max(dim=-1).values
+    bound = tolerance(dtype, 2e-5, 4e-2) * max(1.0, float(want.abs().max()))
+    # (bfloat16: a row whose two best choice scores are within rounding of each other may take the other expert.)
+    allowed = 0 if dtype != torch.bfloat16 else max(1, tokens // 50)
+    assert int((err > bound).sum()) <= allowed, f"{int((err > bound).sum())} rows off by up to {float(err.max())}"
+
+
+@pytest.mark.parametrize("backend", BACKENDS)
+@pytest.mark.parametrize("width", [40, 64, 52, 200, 2050])
+def test_the_norm_with_a_weight_around_zero_over_a_pair_of_outputs(backend, width):
+    """The layer's norm takes the mixer's and the feed-forward's outputs, adds both to the float32 stream and
+    normalises the sum with the scale 1 + w."""
+    from tokenizer_amd.parts import NORMS, NormSpec, Runtime, SumDelta
+    ops, device, dtype = ops_for(backend)
+    gen = torch.Generator().manual_seed(width)
+    rand = lambda *shape: torch.randn(*shape, generator=gen, dtype=torch.float64)
+    stream, first, second, weight = rand(11, width).float().double() * 3, rounded(rand(11, width), dtype), rounded(rand(11, width), dtype), \
+        (rand(width) * 0.2).float().double()
+    spec = NormSpec("rmsnorm", width, 1e-5, options={"tensor_name": "", "offset": 1.0})
+    norm = NORMS.get("rmsnorm")(spec, {"": weight.float().to(device)}, Runtime(dtype, device, ops))
+    residual = stream.float().to(device)
+    delta = SumDelta(ops, first.to(dtype).to(device), second.to(dtype).to(device))
+    out = norm.apply(residual, delta).double().cpu()
+    total = stream + first + second
+    assert float((residual.double().cpu() - total).abs().max()) <= 1e-5
+    want = plain.offset_norm(total, weight, 1e-5)
+    assert float((out - want).abs().max()) <= tolerance(dtype, 1e-5, 2e-2) * max(1.0, float(want.abs().max()))
