@@ -18,7 +18,7 @@ share a prefix of 1,024 ids, with the prefix cache) and prints one JSON line for
 
 times the prompt attention kernel alone on a portion of TOKENS tokens after C cached ones.
 
-    python bench.py --design napadra|dolidra [--size 0.5b|1.5b|7b] [--layers N] [--batch B] [--steps K]
+    python bench.py --design napadra|dolidra|bokulorn [--size 0.5b|1.5b|7b] [--layers N] [--batch B] [--steps K]
 
 times a prefill of 2,048 tokens and decoding at batch B of a Napadra model whose layers have the sizes of the
 Qwen2.5 model named (width, heads, feed-forward and vocabulary; its layers alternate attention, attention on the
@@ -298,16 +298,50 @@ def dolidra_config(sizes: dict, layers: int, window: int = 4096, keep_first: int
             "token_side": {"dim": 16}, "loop": loop, "layers": out}
 
 
+def bokulorn_config(sizes: dict, layers: int, experts: int = 8, top: int = 2) -> dict:
+    """A Bokulorn configuration with the layer sizes of a Qwen2 one.  The layers go round delta rule, latent attention
+    with a rotated key part, latent attention without positions; heads and their sizes are Qwen2's; the cached latent
+    (with the rotated part) is as wide as two of Qwen2's key heads; every layer has a routed feed-forward of `experts`
+    ungated experts of three quarters of the dense inner width, of which a token uses `top` (as many multiply-adds a
+    token as the gated dense one), in four groups of which two are kept."""
+    width, heads, kv_heads = sizes["hidden_size"], sizes["num_attention_heads"], sizes["num_key_value_heads"]
+    d, inner = width // heads, sizes["intermediate_size"]
+    mlp = {"kind": "moe", "expert": {"ff": inner * 3 // 4 // 8 * 8},
+           "router": {"experts": experts, "top": top, "groups": {"count": 4, "keep": 2}}}
+    q_rank = max(64, width // 2 // 64 * 64)
+    out = []
+    for index in range(layers):
+        kind = index % 3
+        if kind == 0:
+            out.append({"type": "channel_delta", "mlp": mlp,
+                        "mixer": {"heads": heads, "kv_heads": kv_heads, "dim": d, "vdim": d, "conv": 4}})
+        elif kind == 1:
+            out.append({"type": "latent_attention", "mlp": mlp,
+                        "mixer": {"heads": heads, "dim": d, "rot_dim": d // 2, "vdim": d, "q_rank": q_rank,
+                                  "kv_rank": 2 * d - d // 2, "scale": (d + d // 2) ** -0.5,
+                                  "rot": {"dims": d // 2, "base": float(sizes.get("rope_theta", 1e6))}}})
+        else:
+            out.append({"type": "latent_attention_2", "mlp": mlp,
+                        "mixer": {"heads": heads, "dim": d, "vdim": d, "q_rank": q_rank, "kv_rank": 2 * d, "scale": d ** -0.5}})
+    return {"architecture": "Bokulorn", "vocab": sizes["vocab_size"], "width": width, "norm": {"eps": 1e-6},
+            "embedding": {"scale": 1.0}, "layers": out}
+
+
 def run_design(args, sizes: dict) -> dict:
-    """Prefill and decode throughput of the named design beside Qwen2 at equal layer sizes and number of layer runs."""
+    """Prefill and decode throughput of the named design beside its closest neighbour (Qwen2; for Bokulorn, Dolidra, whose
+    layers also mix attention with routed experts) at equal layer sizes and number of layer runs."""
     import torch
-    from tokenizer_amd.config import DolidraConfig, NapadraConfig, Qwen2Config
+    from tokenizer_amd.config import BokulornConfig, DolidraConfig, NapadraConfig, Qwen2Config
     from tokenizer_amd.engine import random_model
     layers = args.layers or 8
     steps = min(args.steps, 256)
-    record = {"design": args.design, "beside": "qwen2", "size": args.size, "layers": layers, "dtype": args.dtype,
+    beside = "dolidra" if args.design == "bokulorn" else "qwen2"
+    record = {"design": args.design, "beside": beside, "size": args.size, "layers": layers, "dtype": args.dtype,
               "prompt_len": PROMPT_LEN, "batch": args.batch, "decode_steps": steps, "data": "synthetic (random weights)"}
-    if args.design == "dolidra":
+    if args.design == "bokulorn":
+        configs = {"bokulorn": lambda: BokulornConfig.from_dict(bokulorn_config(sizes, layers)),
+                   "dolidra": lambda: DolidraConfig.from_dict(dolidra_config(sizes, max(2, layers - 2)))}
+    elif args.design == "dolidra":
         # (Two of the layers run twice: `layers` counts the runs, so that both models run as many layers a token.)
         configs = {"dolidra": lambda: DolidraConfig.from_dict(dolidra_config(sizes, max(2, layers - 2))),
                    "qwen2": lambda: Qwen2Config.from_dict(dict(sizes, num_hidden_layers=layers))}
@@ -328,9 +362,9 @@ def run_design(args, sizes: dict) -> dict:
         log(f"{name}: {record[name]}")
         del model
         torch.cuda.empty_cache()
-    if args.design in record and "qwen2" in record:
-        record["prefill_ratio"] = round(record[args.design]["prefill_tokens_per_s"] / record["qwen2"]["prefill_tokens_per_s"], 3)
-        record["decode_ratio"] = round(record[args.design]["decode_tokens_per_s"] / record["qwen2"]["decode_tokens_per_s"], 3)
+    if args.design in record and beside in record:
+        record["prefill_ratio"] = round(record[args.design]["prefill_tokens_per_s"] / record[beside]["prefill_tokens_per_s"], 3)
+        record["decode_ratio"] = round(record[args.design]["decode_tokens_per_s"] / record[beside]["decode_tokens_per_s"], 3)
     return record
 
 
@@ -425,9 +459,9 @@ def main() -> int:
     parser.add_argument("--layers", type=int, default=None)
     parser.add_argument("--size", default="0.5b", choices=["0.5b", "1.5b", "7b"],
                         help="layer sizes of the decode benchmark (the default is the one the record is for)")
-    parser.add_argument("--design", default=None, choices=["napadra", "dolidra"],
-                        help="time this design beside Qwen2 at equal layer sizes (prefill and decode)")
-    parser.add_argument("--only", default=None, choices=["napadra", "dolidra", "qwen2"], help="with --design: one of the two models")
+    parser.add_argument("--design", default=None, choices=["napadra", "dolidra", "bokulorn"],
+                        help="time this design beside its closest neighbour at equal layer sizes (prefill and decode)")
+    parser.add_argument("--only", default=None, choices=["napadra", "dolidra", "bokulorn", "qwen2"], help="with --design: one of the two models")
     parser.add_argument("--peaks", action="store_true", help="measure what the device reaches in HBM reads and bf16 products")
     parser.add_argument("--workload", default=None, choices=["mixed-1.5b", "mixed-0.5b", "prefix-7b"],
                         help="run a serving workload through the scheduler instead of the decode benchmark")

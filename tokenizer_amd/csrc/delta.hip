@@ -86,6 +86,44 @@ short_conv_keep_kernel(const T* __restrict__ rows, int row_stride, ConvRuns runs
   }
 }
 
+// What the recurrence needs of a token that does not depend on the state, for every token side by side: q and k as unit
+// vectors per query/key head (q times d^(-1/2)) and their product, the decays g = exp(neg_rate * softplus(z)) in place
+// of their pre-activations z, and beta = sigmoid(.).  A workgroup a token; a wave a query/key head at a time.
+// prep: float rows of 2 groups d + heads + groups: [q | k | beta | q . k].
+template <typename T>
+__global__ void __launch_bounds__(4 * WAVE)
+delta_prepare_kernel(const T* __restrict__ fresh, int fresh_stride, float* __restrict__ z, const float* __restrict__ neg_rate,
+                     const T* __restrict__ beta_rows, int beta_stride, int beta_offset, float* __restrict__ prep, int heads,
+                     int groups, int d, float unit_eps) {
+  const int t = blockIdx.x, tid = threadIdx.x, lane = tid & (WAVE - 1), wave = tid / WAVE;
+  const int width = 2 * groups * d + heads + groups;
+  const T* x = fresh + (size_t)t * fresh_stride;
+  float* out = prep + (size_t)t * width;
+  const float q_scale = 1.0f / sqrtf((float)d);
+  for (int g = wave; g < groups; g += 4) {
+    float sq = 0.f, sk = 0.f, qk = 0.f;
+    for (int j = lane; j < d; j += WAVE) {
+      const float qv = ld(x + (size_t)g * d + j), kv = ld(x + (size_t)(groups + g) * d + j);
+      sq = fmaf(qv, qv, sq);
+      sk = fmaf(kv, kv, sk);
+      qk = fmaf(qv, kv, qk);
+    }
+    sq = wave_sum(sq);
+    sk = wave_sum(sk);
+    qk = wave_sum(qk);
+    const float inv_q = q_scale / sqrtf(sq + unit_eps), inv_k = 1.0f / sqrtf(sk + unit_eps);
+    for (int j = lane; j < d; j += WAVE) {
+      out[(size_t)g * d + j] = ld(x + (size_t)g * d + j) * inv_q;
+      out[(size_t)(groups + g) * d + j] = ld(x + (size_t)(groups + g) * d + j) * inv_k;
+    }
+    if (lane == 0) out[2 * groups * d + heads + g] = qk * inv_q * inv_k;
+  }
+  float* zt = z + (size_t)t * heads * d;
+  for (int i = tid; i < heads * d; i += 4 * WAVE) zt[i] = expf(neg_rate[i / d] * dl_softplus(zt[i]));
+  for (int h = tid; h < heads; h += 4 * WAVE)
+    out[2 * groups * d + h] = 1.0f / (1.0f + expf(-ld(beta_rows + (size_t)t * beta_stride + beta_offset + h)));
+}
+
 // One workgroup of four waves per (portion, head, 16 columns of S).  A wave owns four columns; its lanes are (column,
 // part p = lane % 16): lane (c, p) keeps rows p PER .. p PER + PER - 1 of column c in registers.  Columns of S do not
 // depend on each other: for column c, with s = g * S[:, c] (row by row), a = k . s and b = q . s (sums within a row of
@@ -94,10 +132,14 @@ short_conv_keep_kernel(const T* __restrict__ rows, int row_stride, ConvRuns runs
 // into LDS sixteen tokens at a time; the next sixteen are asked for before the current ones are worked on.
 // fresh: rows of `fresh_stride`, [groups d (q) | groups d (k) | heads dv (v)]; z: float rows [heads d]; beta's
 // pre-activation at beta_rows[t, beta_offset + h].  A portion that starts at position 0 starts from zeros.
-template <typename T, int PER>
+// PREPARED: `delta_prepare_kernel` has run; z holds the decays themselves and `prep` the unit vectors, beta and q . k,
+// so that between the trips to memory a workgroup does nothing but the recurrence (long portions: the chain from token
+// to token is what bounds them).
+template <typename T, int PER, bool PREPARED>
 __global__ void __launch_bounds__(4 * WAVE)
 delta_scan_kernel(const T* __restrict__ fresh, int fresh_stride, const float* __restrict__ z, const float* __restrict__ neg_rate,
-                  const T* __restrict__ beta_rows, int beta_stride, int beta_offset, float* __restrict__ state,
+                  const float* __restrict__ prep, const T* __restrict__ beta_rows, int beta_stride, int beta_offset,
+                  float* __restrict__ state,
                   size_t state_stride, const int* __restrict__ cu_q, const int* __restrict__ first_position,
                   const int* __restrict__ state_slots, float* __restrict__ out, int heads, int groups, int d, int dv,
                   float unit_eps) {
@@ -120,8 +162,9 @@ delta_scan_kernel(const T* __restrict__ fresh, int fresh_stride, const float* __
     const int j = part * PER + r;
     S[r] = (!from_zero && live && j < d) ? mem[(size_t)j * dv + c] : 0.f;
   }
-  const float rate = neg_rate[h], q_scale = 1.0f / sqrtf((float)d);
-  float q_next[PIECES], k_next[PIECES], g_next[PIECES], v_next = 0.f, beta_next = 0.f;
+  const float rate = PREPARED ? 0.f : neg_rate[h], q_scale = 1.0f / sqrtf((float)d);
+  const int prep_width = 2 * groups * d + heads + groups;
+  float q_next[PIECES], k_next[PIECES], g_next[PIECES], v_next = 0.f, beta_next = 0.f, qk_next = 0.f;
   auto fetch = [&](int t0) {
 #pragma unroll
     for (int i = 0; i < PIECES; ++i) {
@@ -129,9 +172,15 @@ delta_scan_kernel(const T* __restrict__ fresh, int fresh_stride, const float* __
       q_next[i] = k_next[i] = 0.f;
       g_next[i] = 0.f;                               // (a pre-activation; rows past d and tokens past the end get decay 1 below)
       if (j < d && t0 + tok < hi) {
-        const T* x = fresh + (size_t)(t0 + tok) * fresh_stride;
-        q_next[i] = ld(x + (size_t)qk_head * d + j);
-        k_next[i] = ld(x + (size_t)(groups + qk_head) * d + j);
+        if constexpr (PREPARED) {
+          const float* x = prep + (size_t)(t0 + tok) * prep_width;
+          q_next[i] = x[(size_t)qk_head * d + j];
+          k_next[i] = x[(size_t)(groups + qk_head) * d + j];
+        } else {
+          const T* x = fresh + (size_t)(t0 + tok) * fresh_stride;
+          q_next[i] = ld(x + (size_t)qk_head * d + j);
+          k_next[i] = ld(x + (size_t)(groups + qk_head) * d + j);
+        }
         g_next[i] = z[(size_t)(t0 + tok) * heads * d + (size_t)h * d + j];
       }
     }
@@ -140,7 +189,15 @@ delta_scan_kernel(const T* __restrict__ fresh, int fresh_stride, const float* __
       v_next = (col < dv && t0 + tok < hi)
           ? ld(fresh + (size_t)(t0 + tok) * fresh_stride + (size_t)2 * groups * d + (size_t)h * dv + col) : 0.f;
     }
-    if (tid < DL_GROUP) beta_next = t0 + tid < hi ? ld(beta_rows + (size_t)(t0 + tid) * beta_stride + beta_offset + h) : 0.f;
+    if constexpr (PREPARED) {
+      if (tid < DL_GROUP && t0 + tid < hi) {
+        const float* x = prep + (size_t)(t0 + tid) * prep_width + 2 * groups * d;
+        beta_next = x[h];
+        qk_next = x[heads + qk_head];
+      }
+    } else {
+      if (tid < DL_GROUP) beta_next = t0 + tid < hi ? ld(beta_rows + (size_t)(t0 + tid) * beta_stride + beta_offset + h) : 0.f;
+    }
   };
   fetch(lo);
   for (int t0 = lo; t0 < hi; t0 += DL_GROUP) {
@@ -150,14 +207,22 @@ delta_scan_kernel(const T* __restrict__ fresh, int fresh_stride, const float* __
       const int idx = i * 4 * WAVE + tid, tok = idx / DP, j = idx % DP;
       q_s[tok][j] = q_next[i];
       k_s[tok][j] = k_next[i];
-      g_s[tok][j] = (j < d && t0 + tok < hi) ? expf(rate * dl_softplus(g_next[i])) : 1.f;
+      if constexpr (PREPARED) g_s[tok][j] = (j < d && t0 + tok < hi) ? g_next[i] : 1.f;
+      else g_s[tok][j] = (j < d && t0 + tok < hi) ? expf(rate * dl_softplus(g_next[i])) : 1.f;
     }
     v_s[tid >> 4][tid & 15] = v_next;
-    if (tid < DL_GROUP) beta_s[tid] = t0 + tid < hi ? 1.0f / (1.0f + expf(-beta_next)) : 0.f;
+    if constexpr (PREPARED) {
+      if (tid < DL_GROUP) {
+        beta_s[tid] = t0 + tid < hi ? beta_next : 0.f;
+        qk_s[tid] = t0 + tid < hi ? qk_next : 0.f;
+      }
+    } else {
+      if (tid < DL_GROUP) beta_s[tid] = t0 + tid < hi ? 1.0f / (1.0f + expf(-beta_next)) : 0.f;
+    }
     if (t0 + DL_GROUP < hi) fetch(t0 + DL_GROUP);
     __syncthreads();
     // Unit vectors: sixteen threads a token add up the squares (and q . k) over the rows, then scale the rows in place.
-    {
+    if constexpr (!PREPARED) {
       const int tok = tid >> 4, p = tid & 15;
       float sq = 0.f, sk = 0.f, qk = 0.f;
 #pragma unroll
@@ -177,8 +242,8 @@ delta_scan_kernel(const T* __restrict__ fresh, int fresh_stride, const float* __
         k_s[tok][p + 16 * r] *= inv_k;
       }
       if (p == 0) qk_s[tok] = qk * inv_q * inv_k;
+      __syncthreads();
     }
-    __syncthreads();
     // Token by token.  (A token past the portion's end has decay 1, beta 0 and zeros for q, k and v: it changes nothing.
     // Rows past d hold zeros in q and k and decay 1: they stay zero and add nothing.)
     float read[DL_GROUP];
@@ -239,24 +304,40 @@ extern "C" int ta_short_conv_silu(const void* rows, int row_stride, int o0, int 
 }
 
 // fresh: rows of `fresh_stride` elements, [groups d (q) | groups d (k) | heads dv (v)]; z float [n_tokens, heads d];
-// neg_rate float [heads]; out float [n_tokens, heads dv].
-extern "C" int ta_delta_scan(const void* fresh, int fresh_stride, const void* z, const void* neg_rate, const void* beta_rows,
+// neg_rate float [heads]; out float [n_tokens, heads dv].  prep: null, or room for n_tokens rows of
+// 2 groups d + heads + groups floats: then what does not depend on the state is made for all tokens side by side first
+// (z then holds the decays afterwards), which is what steps with long portions want.
+extern "C" int ta_delta_scan(const void* fresh, int fresh_stride, void* z, const void* neg_rate, const void* beta_rows,
                              int beta_stride, int beta_offset, void* state, long state_stride, const void* cu_q,
-                             const void* first_position, const void* state_slots, void* out, int n_entries, int heads,
-                             int groups, int d, int dv, float unit_eps, int dtype, hipStream_t stream) {
-  if (n_entries <= 0) return 0;
+                             const void* first_position, const void* state_slots, void* out, void* prep, int n_tokens,
+                             int n_entries, int heads, int groups, int d, int dv, float unit_eps, int dtype,
+                             hipStream_t stream) {
+  if (n_entries <= 0 || n_tokens <= 0) return 0;
   if (d < 1 || d > DL_MAX_D || dv < 1 || heads < 1 || groups < 1 || heads % groups || heads > 65535 ||
       state_stride < (long)heads * d * dv)
     return -1;
   dim3 grid(n_entries, heads, (dv + 15) / 16);
   if (grid.z > 65535) return -1;
   const int per = (d + 15) / 16;
-#define SCAN(TT, PP) delta_scan_kernel<TT, PP><<<grid, 4 * WAVE, 0, stream>>>((const TT*)fresh, fresh_stride, (const float*)z, \
-    (const float*)neg_rate, (const TT*)beta_rows, beta_stride, beta_offset, (float*)state, (size_t)state_stride,             \
-    (const int*)cu_q, (const int*)first_position, (const int*)state_slots, (float*)out, heads, groups, d, dv, unit_eps)
-#define SCANS(TT) if (per <= 1) SCAN(TT, 1); else if (per <= 2) SCAN(TT, 2); else if (per <= 4) SCAN(TT, 4);                 \
-                  else if (per <= 8) SCAN(TT, 8); else SCAN(TT, 16)
-  if (dtype == DT_F32) { SCANS(float); } else { SCANS(bf16_t); }
+  if (prep) {
+    if (dtype == DT_F32)
+      delta_prepare_kernel<float><<<n_tokens, 4 * WAVE, 0, stream>>>((const float*)fresh, fresh_stride, (float*)z,
+          (const float*)neg_rate, (const float*)beta_rows, beta_stride, beta_offset, (float*)prep, heads, groups, d, unit_eps);
+    else
+      delta_prepare_kernel<bf16_t><<<n_tokens, 4 * WAVE, 0, stream>>>((const bf16_t*)fresh, fresh_stride, (float*)z,
+          (const float*)neg_rate, (const bf16_t*)beta_rows, beta_stride, beta_offset, (float*)prep, heads, groups, d, unit_eps);
+  }
+#define SCAN(TT, PP, RR) delta_scan_kernel<TT, PP, RR><<<grid, 4 * WAVE, 0, stream>>>((const TT*)fresh, fresh_stride,        \
+    (const float*)z, (const float*)neg_rate, (const float*)prep, (const TT*)beta_rows, beta_stride, beta_offset,             \
+    (float*)state, (size_t)state_stride, (const int*)cu_q, (const int*)first_position, (const int*)state_slots,             \
+    (float*)out, heads, groups, d, dv, unit_eps)
+#define SCANS(TT, RR) if (per <= 1) SCAN(TT, 1, RR); else if (per <= 2) SCAN(TT, 2, RR); else if (per <= 4) SCAN(TT, 4, RR); \
+                      else if (per <= 8) SCAN(TT, 8, RR); else SCAN(TT, 16, RR)
+  if (prep) {
+    if (dtype == DT_F32) { SCANS(float, true); } else { SCANS(bf16_t, true); }
+  } else {
+    if (dtype == DT_F32) { SCANS(float, false); } else { SCANS(bf16_t, false); }
+  }
 #undef SCANS
 #undef SCAN
   return LAUNCH_STATUS();

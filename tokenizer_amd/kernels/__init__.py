@@ -403,7 +403,11 @@ class Ops:
         dv); q and k become unit vectors, x / sqrt(sum x^2 + unit_eps), q times d^(-1/2).  decay float32 [T, heads d]:
         g = exp(neg_rate[h] * softplus(decay)); beta = sigmoid(rows[t, beta_offset + h]).  Per head and token:
         S <- diag(g) S; u = beta (v - S^T k); S <- S + k u^T; out = S^T q.  state float32 [slots, >= heads d dv] (an
-        entry whose first position is 0 starts from zeros); out float32 [T, heads dv]."""
+        entry whose first position is 0 starts from zeros); out float32 [T, heads dv].
+
+        Steps with portions of many rows (more than `DELTA_PREPARE_ROWS` rows an entry on average) first make what does
+        not depend on the state for all tokens side by side (unit vectors, q . k, beta and the decays, which then stand in
+        `decay` in place of their pre-activations), so that the walk from token to token does nothing else."""
         _dev(fresh, decay, neg_rate, rows, state, cu_q, first_position, state_slots, out)
         n_tokens = fresh.shape[0]
         _need(heads > 0 and groups > 0 and heads % groups == 0 and 0 < d <= 256 and dv > 0, "heads of up to 256 key channels")
@@ -416,11 +420,18 @@ class Ops:
         _need(out.dtype == torch.float32 and tuple(out.shape) == (n_tokens, heads * dv), "out float32 [T, heads dv]")
         n_entries = cu_q.numel() - 1
         _need(first_position.numel() == n_entries == state_slots.numel(), "one first position and slot per entry")
+        prepared = None
+        if n_tokens > self.DELTA_PREPARE_ROWS * n_entries:
+            _need(decay.is_contiguous(), "the decays' rows are written in place")
+            prepared = torch.empty((n_tokens, 2 * groups * d + heads + groups), dtype=torch.float32, device=fresh.device)
         self._check(self.lib.ta_delta_scan(_ptr(fresh), fresh.shape[1], _ptr(decay), _ptr(neg_rate), _ptr(rows), rows.shape[1],
                                            beta_offset, _ptr(state), ctypes.c_long(state.shape[1]), _ptr(cu_q),
-                                           _ptr(first_position), _ptr(state_slots), _ptr(out), n_entries, heads, groups, d, dv,
-                                           ctypes.c_float(unit_eps), _code(fresh.dtype), self._stream()), "delta_scan")
+                                           _ptr(first_position), _ptr(state_slots), _ptr(out), _ptr(prepared), n_tokens,
+                                           n_entries, heads, groups, d, dv, ctypes.c_float(unit_eps), _code(fresh.dtype),
+                                           self._stream()), "delta_scan")
         return out
+
+    DELTA_PREPARE_ROWS = 4     # rows an entry (on average) above which the delta rule's inputs are prepared side by side
 
     # ---------------------------------------------------- sigmoid router with groups, ungated experts
     def route_sigmoid(self, logits: torch.Tensor, correction: torch.Tensor, n_groups: int, keep_groups: int,
@@ -1070,6 +1081,11 @@ class Ops:
         costs no launch, and a K from 512 on is cut as well, into parts of at least 224 (the output projection of
         a decode batch: every workgroup reads all the rows, and a quarter of K is a quarter of them)."""
         shortest, part = (self.PENDING_SHORTEST_K, 224) if pending else (2048, 512)
+        if self.use_split_k and 0 < m <= self.FUSED_ROWS and k >= self.FEW_ROWS_LONG_K and n % 4 == 0 and -(-n // 16) < 128:
+            # Up to sixteen rows, a very long K and few output columns (the down product over all experts of a routed
+            # layer in a decode step: K is experts times the inner width): one workgroup a tile of sixteen columns would
+            # leave most compute units without a share of the weights.
+            return max(1, min(-(-self.compute_units // -(-n // 16)), k // 2048))
         if (not self.use_split_k or not (self.FUSED_ROWS < m <= self.SKINNY_ROWS) or n % 4
                 or not (shortest <= k < self.SPLIT_K_FROM)):
             return 1
@@ -1080,6 +1096,7 @@ class Ops:
             tiles = -(-n // 32)        # more than 32 rows: a workgroup takes two blocks of sixteen columns
         return max(1, min(-(-self.compute_units // tiles), k // part))
 
+    FEW_ROWS_LONG_K = 8192     # the shortest K that is cut for up to sixteen rows
     PENDING_SHORTEST_K = 512   # the shortest K that is cut when the parts may be left for the next norm
     SPLIT_K_FROM = 8192        # the shortest K that the tiled kernel cuts (shorter ones are the weight-streaming kernel's)
 
