@@ -334,24 +334,12 @@ extern "C" int ta_gelu_gate(const void* in, void* out, int n_tokens, int inner, 
 // one score if it has one expert), and experts outside the `keep` best groups (the lower index of equals) count as minus
 // infinity.  The `top` largest choice scores (the lower index of equals) are chosen, in falling order; their weights
 // are their s over the sum of the chosen s (+ 1e-20).  A wave a token; the scores of a token lie in LDS.
-__global__ void __launch_bounds__(256)
-route_sigmoid_kernel(const float* __restrict__ logits, const float* __restrict__ correction, int n_tokens, int n_experts,
-                     int n_groups, int keep, int top, int* __restrict__ chosen, float* __restrict__ weights) {
-  extern __shared__ float rs_scratch[];
-  const int lane = threadIdx.x & (WAVE - 1), wave = threadIdx.x / WAVE;
-  const int slot = blockIdx.x * (blockDim.x / WAVE) + wave;
-  const bool live = slot < n_tokens;                          // (a wave past the end works on the last token and stores nothing)
-  const int t = live ? slot : n_tokens - 1;
-  float* choice = rs_scratch + (size_t)wave * (2 * n_experts + n_groups);
-  float* score = choice + n_experts;
-  float* worth = score + n_experts;
-  const float* row = logits + (size_t)t * n_experts;
-  for (int e = lane; e < n_experts; e += WAVE) {
-    const float s = 1.0f / (1.0f + expf(-row[e]));
-    score[e] = s;
-    choice[e] = s + correction[e];
-  }
-  __syncthreads();
+// The choice among one token's scores in LDS (`choice`: s + correction, `score`: s, `worth`: room for a number a group).
+// Every wave that calls it for a token runs the same steps between the same barriers (waves that share a token write
+// the same values); `store` says whether this wave writes the token's results.
+__device__ __forceinline__ void rs_choose(float* choice, const float* score, float* worth, int lane, int n_experts,
+                                          int n_groups, int keep, int top, bool store, int* __restrict__ chosen_row,
+                                          float* __restrict__ weights_row) {
   if (n_groups > 0) {
     const int per = n_experts / n_groups;
     for (int g = lane; g < n_groups; g += WAVE) {
@@ -397,11 +385,82 @@ route_sigmoid_kernel(const float* __restrict__ logits, const float* __restrict__
     const float s = score[best_at];
     total += s;
     if (lane == k) mine = s;
-    if (live && lane == 0) chosen[(size_t)t * top + k] = best_at;
+    if (store && lane == 0) chosen_row[k] = best_at;
     last = best_at;
     last_value = best;
   }
-  if (live && lane < top) weights[(size_t)t * top + lane] = mine / (total + 1e-20f);
+  if (store && lane < top) weights_row[lane] = mine / (total + 1e-20f);
+}
+
+__global__ void __launch_bounds__(256)
+route_sigmoid_kernel(const float* __restrict__ logits, const float* __restrict__ correction, int n_tokens, int n_experts,
+                     int n_groups, int keep, int top, int* __restrict__ chosen, float* __restrict__ weights) {
+  extern __shared__ float rs_scratch[];
+  const int lane = threadIdx.x & (WAVE - 1), wave = threadIdx.x / WAVE;
+  const int slot = blockIdx.x * (blockDim.x / WAVE) + wave;
+  const bool live = slot < n_tokens;                          // (a wave past the end works on the last token and stores nothing)
+  const int t = live ? slot : n_tokens - 1;
+  float* choice = rs_scratch + (size_t)wave * (2 * n_experts + n_groups);
+  float* score = choice + n_experts;
+  float* worth = score + n_experts;
+  const float* row = logits + (size_t)t * n_experts;
+  for (int e = lane; e < n_experts; e += WAVE) {
+    const float s = 1.0f / (1.0f + expf(-row[e]));
+    score[e] = s;
+    choice[e] = s + correction[e];
+  }
+  __syncthreads();
+  rs_choose(choice, score, worth, lane, n_experts, n_groups, keep, top, live, chosen + (size_t)t * top, weights + (size_t)t * top);
+}
+
+// The router's product and the choice in one kernel, a token a workgroup (few rows: a decode step): as route_rows_kernel
+// forms the logits (float sums of the row with each expert's router row, the row kept in registers), then all four
+// waves choose together and the first stores.
+template <typename T>
+__global__ void __launch_bounds__(256)
+route_rows_sigmoid_kernel(const T* __restrict__ x, int lda, const T* __restrict__ router, const float* __restrict__ correction,
+                          int hidden, int n_experts, int n_groups, int keep, int top, int* __restrict__ chosen,
+                          float* __restrict__ weights) {
+  constexpr int N = RtVec<T>::N;
+  extern __shared__ float rs_scratch[];
+  float* choice = rs_scratch;
+  float* score = choice + n_experts;
+  float* worth = score + n_experts;
+  const int t = blockIdx.x;
+  const int lane = threadIdx.x & (WAVE - 1), wave = threadIdx.x / WAVE;
+  const T* row = x + (size_t)t * lda;
+  float xv[RT_ROW_PIECES][N];
+#pragma unroll
+  for (int p = 0; p < RT_ROW_PIECES; ++p) {
+    const int at = (p * WAVE + lane) * N;
+    if (at < hidden) RtVec<T>::load(row + at, xv[p]);
+    else
+#pragma unroll
+      for (int k = 0; k < N; ++k) xv[p][k] = 0.f;
+  }
+  for (int e = wave; e < n_experts; e += 256 / WAVE) {
+    const T* w = router + (size_t)e * hidden;
+    float sum = 0.f;
+#pragma unroll
+    for (int p = 0; p < RT_ROW_PIECES; ++p) {
+      const int at = (p * WAVE + lane) * N;
+      if (at < hidden) {
+        float wv[N];
+        RtVec<T>::load(w + at, wv);
+#pragma unroll
+        for (int k = 0; k < N; ++k) sum = fmaf(wv[k], xv[p][k], sum);
+      }
+    }
+    sum = wave_sum(sum);
+    if (lane == 0) {
+      const float s = 1.0f / (1.0f + expf(-sum));
+      score[e] = s;
+      choice[e] = s + correction[e];
+    }
+  }
+  __syncthreads();
+  rs_choose(choice, score, worth, lane, n_experts, n_groups, keep, top, wave == 0, chosen + (size_t)t * top,
+            weights + (size_t)t * top);
 }
 
 // up: [n_tokens, n_experts * inner]; out: [n_tokens, columns], columns >= n_experts * inner:
@@ -479,6 +538,27 @@ extern "C" int ta_route_sigmoid(const void* logits, const void* correction, int 
   const size_t lds = (size_t)4 * (2 * n_experts + n_groups) * sizeof(float);
   route_sigmoid_kernel<<<(n_tokens + 3) / 4, 256, lds, stream>>>((const float*)logits, (const float*)correction, n_tokens,
                                                                  n_experts, n_groups, keep, top, (int*)chosen, (float*)weights);
+  return LAUNCH_STATUS();
+}
+
+// Returns -2 for sizes the fused kernel does not take (the caller then forms the logits with a product of its own).
+extern "C" int ta_route_rows_sigmoid(const void* x, int lda, const void* router, const void* correction, int n_tokens,
+                                     int hidden, int n_experts, int n_groups, int keep, int top, void* chosen, void* weights,
+                                     int dtype, hipStream_t stream) {
+  if (n_tokens <= 0) return 0;
+  if (top <= 0 || top > n_experts || top > WAVE || n_groups < 0) return -1;
+  if (n_groups > 0 && (n_experts % n_groups || keep <= 0 || keep > n_groups || keep * (n_experts / n_groups) < top)) return -1;
+  const int piece = dtype == DT_F32 ? 4 : 8;
+  if (n_experts > RT_MAX_EXPERTS || hidden % piece || lda % piece || hidden > WAVE * RT_ROW_PIECES * piece ||
+      (((uintptr_t)x | (uintptr_t)router) & 15))
+    return -2;
+  const size_t lds = (size_t)(2 * n_experts + n_groups) * sizeof(float);
+  if (dtype == DT_F32)
+    route_rows_sigmoid_kernel<float><<<n_tokens, 256, lds, stream>>>((const float*)x, lda, (const float*)router,
+        (const float*)correction, hidden, n_experts, n_groups, keep, top, (int*)chosen, (float*)weights);
+  else
+    route_rows_sigmoid_kernel<bf16_t><<<n_tokens, 256, lds, stream>>>((const bf16_t*)x, lda, (const bf16_t*)router,
+        (const float*)correction, hidden, n_experts, n_groups, keep, top, (int*)chosen, (float*)weights);
   return LAUNCH_STATUS();
 }
 

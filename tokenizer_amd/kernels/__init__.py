@@ -157,7 +157,7 @@ class Ops:
                      "ta_capped_gate", "ta_norm_add_rmsnorm", "ta_norm_rotate_store", "ta_differential_heads",
                      "ta_sigmoid_head_gate", "ta_route_top", "ta_expert_gate", "ta_side_gate", "ta_gelu_gate", "ta_norm_side_norm", "ta_route_rows", "ta_expert_slots", "ta_grouped_gemm_bf16", "ta_expert_combine",
                      "ta_add_pair_rmsnorm", "ta_latent_store", "ta_rotate_tails", "ta_head_linear", "ta_short_conv_silu",
-                     "ta_delta_scan", "ta_route_sigmoid", "ta_expert_act", "ta_relu2"):
+                     "ta_delta_scan", "ta_route_sigmoid", "ta_route_rows_sigmoid", "ta_expert_act", "ta_relu2"):
             getattr(self.lib, name).restype = ctypes.c_int
         self.lib.ta_grouped_gemm_bf16.argtypes = [ctypes.c_void_p, ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int,
                                                   ctypes.c_int, ctypes.c_void_p, ctypes.c_long, ctypes.c_int, ctypes.c_void_p,
@@ -625,6 +625,32 @@ class Ops:
         self._check(status, "route_rows")
         return True
 
+    def route_rows_sigmoid(self, x: torch.Tensor, router: torch.Tensor, correction: torch.Tensor, n_groups: int,
+                           keep_groups: int, chosen: torch.Tensor, weights: torch.Tensor) -> bool:
+        """`route_sigmoid` of the float32 logits x @ router.T without leaving them in memory: product and choice in one
+        kernel, a token a workgroup (for the few rows of a decode step).  Returns False for sizes the kernel does not take
+        (as `route_rows`): the caller then forms the logits with `linear` and calls `route_sigmoid`."""
+        _dev(x, router, correction, chosen, weights)
+        n_tokens, hidden = x.shape
+        n_experts, top = router.shape[0], chosen.shape[1]
+        _need(x.dtype == router.dtype and x.stride(1) == 1 and router.is_contiguous() and router.shape[1] == hidden, "router [E, H]")
+        _need(correction.dtype == torch.float32 and correction.numel() == n_experts, "the correction is float32 [E]")
+        _need(chosen.dtype == torch.int32 and weights.dtype == torch.float32 and chosen.is_contiguous() and weights.is_contiguous()
+              and tuple(chosen.shape) == (n_tokens, top) == tuple(weights.shape), "chosen int32 and weights float32 [T, top]")
+        _need(0 < top <= min(n_experts, 64), "between one and 64 experts a token, no more than there are")
+        _need(n_groups >= 0 and (n_groups == 0 or (n_experts % n_groups == 0 and 0 < keep_groups <= n_groups
+                                                   and keep_groups * (n_experts // n_groups) >= top)),
+              "the kept groups must hold the experts a token uses")
+        status = self.lib.ta_route_rows_sigmoid(_ptr(x), x.stride(0) if n_tokens > 1 else hidden, _ptr(router), _ptr(correction),
+                                                n_tokens, hidden, n_experts, n_groups, keep_groups, top, _ptr(chosen),
+                                                _ptr(weights), _code(x.dtype), self._stream())
+        if status == -2:
+            return False
+        self._check(status, "route_rows_sigmoid")
+        return True
+
+    ROUTE_ROWS_FUSED = 64      # rows up to which the sigmoid router's product and choice are one kernel (a workgroup a row)
+
     # Routed feed-forwards over sorted tokens (bfloat16): tiles of `bm` slots that belong to one expert each.
     GROUPED_EXPERTS = 256
 
@@ -1085,7 +1111,9 @@ class Ops:
             # Up to sixteen rows, a very long K and few output columns (the down product over all experts of a routed
             # layer in a decode step: K is experts times the inner width): one workgroup a tile of sixteen columns would
             # leave most compute units without a share of the weights.
-            return max(1, min(-(-self.compute_units // -(-n // 16)), k // 2048))
+            # (8 rows x 896 columns over a K of 29,184: 50 us in one piece, 24 in five parts, 19 in eight to twelve; 1,536
+            # columns over 53,760: 95, 45 in five to eight.)
+            return max(1, min(-(-2 * self.compute_units // -(-n // 16)), k // 2048))
         if (not self.use_split_k or not (self.FUSED_ROWS < m <= self.SKINNY_ROWS) or n % 4
                 or not (shortest <= k < self.SPLIT_K_FROM)):
             return 1

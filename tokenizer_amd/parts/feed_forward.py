@@ -175,8 +175,11 @@ class RoutedExperts(FeedForward):
         chosen = torch.empty((x.shape[0], self.top_k), dtype=torch.int32, device=x.device)
         weights = torch.empty((x.shape[0], self.top_k), dtype=torch.float32, device=x.device)
         if self.sigmoid:
-            ops.route_sigmoid(ops.linear(x, self.w_router, out_dtype=torch.float32), self.correction, self.n_groups,
-                              self.keep_groups, chosen, weights)
+            fused = getattr(ops, "route_rows_sigmoid", None)   # few rows: the router's product and the choice in one kernel
+            if (fused is None or x.shape[0] > ops.ROUTE_ROWS_FUSED
+                    or not fused(x, self.w_router, self.correction, self.n_groups, self.keep_groups, chosen, weights)):
+                ops.route_sigmoid(ops.linear(x, self.w_router, out_dtype=torch.float32), self.correction, self.n_groups,
+                                  self.keep_groups, chosen, weights)
         else:
             fused = getattr(ops, "route_rows", None)      # the router's product and the choice in one kernel, where there is one
             if fused is None or not fused(x, self.w_router, chosen, weights):
