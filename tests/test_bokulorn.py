@@ -371,6 +371,7 @@ def latent_tensors(gen, rotated, width, heads, d, dv, q_rank, kv_rank, rot_dim, 
 @pytest.mark.parametrize("rotated,width,heads,d,dv,q_rank,kv_rank,rot_dim,scale,base", [
     (True, 48, 4, 16, 24, 24, 40, 8, 0.3, 10000.0), (True, 40, 3, 10, 14, 20, 22, 6, 0.35, 300.0),
     (True, 32, 1, 24, 40, 16, 30, 2, 0.2, 100.0), (True, 64, 2, 32, 32, 48, 112, 16, 0.18, 500000.0),
+    (True, 64, 2, 16, 16, 32, 288, 32, 0.2, 10000.0),             # a latent wider than any head of keys
     (False, 48, 2, 32, 16, 32, 32, 0, 0.2, 1.0), (False, 40, 3, 6, 10, 12, 18, 0, 0.4, 1.0),
     (False, 64, 4, 16, 64, 64, 96, 0, 0.25, 1.0)])
 def test_latent_attention_alone(backend, cut, rotated, width, heads, d, dv, q_rank, kv_rank, rot_dim, scale, base):

@@ -4,7 +4,7 @@
 #include "common.h"
 
 #define ATT_WAVES 4
-#define ATT_MAX_D 256
+#define ATT_MAX_D 512          // (a cached latent with its rotated part may be wider than any head of keys)
 
 // q: rows of `q_stride` elements, head h at h*d.  out: [n_tokens, n_q*d].
 // Token t at position p of entry e sees keys max(0, p-window)..p (window < 0: all from 0), whose
@@ -46,7 +46,7 @@ paged_attention_generic(const T* __restrict__ q, int q_stride, T* __restrict__ o
   for (int i = threadIdx.x; i < d; i += blockDim.x) q_s[i] = ld(q + (size_t)t * q_stride + (size_t)h * d + i);
   __syncthreads();
 
-  float acc[ATT_MAX_D / WAVE] = {0.f, 0.f, 0.f, 0.f};
+  float acc[ATT_MAX_D / WAVE] = {};
   float m = -INFINITY, l = 0.f;
 
   for (int base = wave * WAVE; base < n_keys; base += ATT_WAVES * WAVE) {

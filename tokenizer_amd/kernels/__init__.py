@@ -852,7 +852,7 @@ class Ops:
         _need(entry_of_token.dtype == torch.int32 and entry_of_token.numel() == n_tokens, "entry_of_token must be int32 [T]")
         _need(block_table.dtype == torch.int32 and block_table.dim() == 2, "block_table must be int32 [E, P]")
         _need(n_kv > 0 and n_q % n_kv == 0, "query heads must be a multiple of kv heads")
-        _need(0 < head_dim <= 256 and 0 < value_dim <= 256, "head sizes up to 256 are supported")
+        _need(0 < head_dim <= 512 and 0 < value_dim <= 512, "head sizes up to 512 are supported")
         if max_position is not None:
             _need(max_position // page_size < block_table.shape[1], "block table is too narrow for the positions")
         # The matrix-core kernels take chunks, slopes and sinks as they are; value heads of another size than the key
