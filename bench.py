@@ -299,7 +299,7 @@ def dolidra_config(sizes: dict, layers: int, window: int = 4096, keep_first: int
 
 
 def bokulorn_config(sizes: dict, layers: int, experts: int = 8, top: int = 2) -> dict:
-    """A Bokulorn configuration with the layer sizes of a Qwen2 one.  The layers go round delta rule, latent attention
+    """A Bokulorn configuration with the layer sizes of a Qwen2 one.  The layers cycle through delta rule, latent attention
     with a rotated key part, latent attention without positions; heads and their sizes are Qwen2's; the cached latent
     (with the rotated part) is as wide as two of Qwen2's key heads; every layer has a routed feed-forward of `experts`
     ungated experts of three quarters of the dense inner width, of which a token uses `top` (as many multiply-adds a

@@ -196,6 +196,17 @@ def test_hundreds_of_tokens(folders, oracle, dtype, cut):
 
 @pytest.mark.gpu
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("cut", ["whole", "tail"])
+def test_a_prompt_of_fifteen_hundred_tokens(folders, oracle, dtype, cut):
+    """All three mixers and layers that share tensors, far beyond one tile of the prompt kernels and one trip of the scan."""
+    name = "A"
+    reqs = requests_for(name, (1500, 70))
+    steps = tt.whole(reqs) if cut == "whole" else tt.decode_tail(reqs, 40)
+    check_trace(folders, oracle, name, f"gpu-{dtype}", steps, reqs)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_the_replay_program_on_a_model_folder(folders, oracle, tmp_path, dtype):
     name = "B"
     reqs = requests_for(name, (40, 23, 5, 64, 31))
@@ -411,6 +422,25 @@ def test_latent_attention_alone(backend, cut, rotated, width, heads, d, dv, q_ra
     if rotated:         # the positions do matter: the same rows with every position one further give other outputs
         shifted = plain.latent_attention(torch.cat([h[:1], h]), m, w, eps, True)[1:]
         assert float((shifted - want).abs().max()) > 0.05
+
+
+@pytest.mark.parametrize("backend", BACKENDS)
+@pytest.mark.parametrize("rotated,heads,d,dv,kv_rank,rot_dim", [(True, 16, 16, 16, 48, 16), (False, 24, 8, 8, 32, 0), (True, 5, 24, 16, 72, 8)])
+def test_many_heads_on_one_latent_over_a_long_prompt(backend, rotated, heads, d, dv, kv_rank, rot_dim):
+    """More query heads on the one cached row than a grouped-query model has on a key head, over 600 tokens: a prompt of
+    300, a single token, a portion of 267 behind them, then single tokens."""
+    ops, device, dtype = ops_for(backend)
+    gen = torch.Generator().manual_seed(heads + kv_rank)
+    width, q_rank, n, eps, scale, base = 64, 40, 600, 1e-6, 0.25, 10000.0
+    w = latent_tensors(gen, rotated, width, heads, d, dv, q_rank, kv_rank, rot_dim, dtype, size=3.0)
+    h = rounded(torch.randn(n, width, generator=gen, dtype=torch.float64), dtype)
+    m = {"heads": heads, "dim": d, "vdim": dv, "kv_rank": kv_rank, "rot_dim": rot_dim, "scale": scale,
+         "rot": {"base": base, "dims": rot_dim}}
+    want = plain.latent_attention(h, m, w, eps, rotated)
+    runner = PartRunner("latent_attention", latent_spec(rotated, width, heads, d, dv, q_rank, kv_rank, rot_dim, scale, base, eps),
+                        w, backend, num_pages=44)
+    got = runner.run(h, [300, 1, 267] + [1] * 32, rider=h[:20] * 0.5)
+    assert float((got - want).abs().max()) <= tolerance(dtype, 3e-5, 5e-2) * max(1.0, float(want.abs().max()))
 
 
 @pytest.mark.parametrize("backend", BACKENDS)
