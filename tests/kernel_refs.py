@@ -81,7 +81,7 @@ class PlainOps:
 
     # ------------------------------------------------------------ delta rule with a decay per key channel
     def short_conv_silu(self, rows, offsets, widths, taps, state, state_offset, cu_q, first_position, state_slots,
-                        entry_of_token, out):
+                        entry_of_token, out, bias=None):
         w = self.work
         n_taps, channels = taps.shape[1], sum(widths)
         x = torch.cat([rows[:, o:o + n] for o, n in zip(offsets, widths)], dim=1).to(w)
@@ -95,11 +95,85 @@ class PlainOps:
                 tail = torch.zeros_like(tail)
             seen = torch.cat([tail, x[lo:hi]], dim=0)
             y = torch.zeros((hi - lo, channels), dtype=w)
+            if bias is not None:
+                y = y + bias.to(w)
             for j in range(n_taps):
                 y = y + seen[j:j + hi - lo] * taps[:, j].to(w)
             out[lo:hi] = (y * torch.sigmoid(y)).to(out.dtype)
             state[slot, state_offset:state_offset + (n_taps - 1) * channels] = seen[seen.shape[0] - (n_taps - 1):].reshape(-1).to(state.dtype)
         return out
+
+    def selective_scan(self, x, pre, neg_rate, low, b_offset, c_offset, skip, rows, z_offset, state, cu_q,
+                       first_position, state_slots, out, channels, n):
+        w = self.work
+        soft = lambda v: torch.where(v > 30.0, v, torch.log1p(torch.exp(torch.clamp(v, max=30.0))))
+        A = neg_rate.to(w)
+        for e in range(cu_q.numel() - 1):
+            lo, hi = int(cu_q[e]), int(cu_q[e + 1])
+            if hi <= lo:
+                continue
+            slot = int(state_slots[e])
+            S = state[slot, :channels * n].to(w).reshape(channels, n)
+            if int(first_position[e]) == 0:
+                S = torch.zeros_like(S)
+            for t in range(lo, hi):
+                step, xt = soft(pre[t].to(w)), x[t].to(w)
+                B, C = low[t, b_offset:b_offset + n].to(w), low[t, c_offset:c_offset + n].to(w)
+                S = torch.exp(step[:, None] * A) * S + (step * xt)[:, None] * B[None, :]
+                y = S @ C + skip.to(w) * xt
+                z = rows[t, z_offset:z_offset + channels].to(w)
+                out[t] = (y * (z * torch.sigmoid(z))).to(out.dtype)
+            state[slot, :channels * n] = S.reshape(-1).to(state.dtype)
+        return out
+
+    def add_terms_rmsnorm(self, residual, terms, weight, eps, out, rows=None, store_residual=True, weight2=None,
+                          eps2=0.0, out2=None):
+        pick = (lambda t: t) if rows is None else (lambda t: t[rows.long()])
+        x = pick(residual).to(self.work)
+        total = None
+        for term, factor, scale in terms:
+            part = pick(term).to(self.work) * factor
+            if scale is not None:
+                part = part * scale.to(self.work)
+            total = part if total is None else total + part
+        if total is not None:
+            x = x + total
+        if store_residual:
+            assert rows is None
+            residual.copy_(x.to(torch.float32))
+            x = residual.to(self.work)
+        unit = lambda e: x / torch.sqrt((x * x).mean(dim=-1, keepdim=True) + e)
+        out.copy_((x if weight is None else unit(eps) * weight.to(self.work)).to(out.dtype))
+        if out2 is not None:
+            out2.copy_((unit(eps2) * weight2.to(self.work)).to(out2.dtype))
+        return out
+
+    def scale_cap(self, x, scale, cap):
+        y = x.to(self.work) * scale
+        if cap:
+            y = cap * torch.tanh(y / cap)
+        x.copy_(y.to(x.dtype))
+        return x
+
+    def route_scores(self, logits, correction, n_experts, n_groups, keep_groups, chosen, weights, softmax=False,
+                     group_max=False, gate=None):
+        top = chosen.shape[1]
+        z = logits.to(torch.float32)
+        s = torch.softmax(z[:, :n_experts], dim=-1) if softmax else torch.sigmoid(z[:, :n_experts])
+        choice = s if correction is None else s + correction.to(torch.float32)
+        if n_groups:
+            per = n_experts // n_groups
+            grouped = choice.reshape(-1, n_groups, per)
+            worth = grouped.max(-1).values if group_max else torch.topk(grouped, min(2, per), dim=-1).values.sum(-1)
+            best = torch.topk(worth, keep_groups, dim=-1).indices
+            allowed = torch.zeros_like(worth, dtype=torch.bool).scatter_(1, best, True)
+            choice = grouped.masked_fill(~allowed[:, :, None], float("-inf")).reshape(choice.shape)
+        ids = torch.topk(choice, top, dim=-1).indices
+        picked = torch.gather(s, 1, ids)
+        chosen.copy_(ids.to(torch.int32))
+        weights.copy_(picked / (picked.sum(-1, keepdim=True) + 1e-20))
+        if gate is not None:
+            gate.copy_(torch.sigmoid(z[:, n_experts]))
 
     def delta_scan(self, fresh, decay, neg_rate, rows, beta_offset, state, cu_q, first_position, state_slots, out,
                    heads, groups, d, dv, unit_eps):
@@ -330,7 +404,7 @@ class PlainOps:
 
     def paged_attention(self, qkv, out, k_pages, v_pages, positions, entry_of_token, block_table,
                         n_q, n_kv, head_dim, window, scale, max_position=None, batch=None,
-                        value_dim=None, chunk=None, slopes=None, sinks=None, keep_first=0, value_heads=None):
+                        value_dim=None, chunk=None, slopes=None, sinks=None, keep_first=0, value_heads=None, softcap=None):
         page_size = k_pages.shape[2]
         group = n_q // n_kv
         share = 1 if value_heads is None else n_kv // value_heads     # key heads that read one value head
@@ -355,6 +429,8 @@ class PlainOps:
             if slopes is not None:
                 distance = pos - torch.tensor(keys, dtype=self.work)
                 scores = scores - slopes.to(self.work)[:, None] * distance[None, :]
+            if softcap:
+                scores = softcap * torch.tanh(scores / softcap)
             if sinks is None:
                 probs = torch.softmax(scores, dim=-1)
             else:
@@ -444,7 +520,7 @@ class PlainOps:
         chosen.copy_(ids.to(torch.int32))
         weights.copy_(torch.softmax(values, dim=-1))
 
-    def expert_gate(self, gate_up, chosen, weights, n_experts, inner, shared, out):
+    def expert_gate(self, gate_up, chosen, weights, n_experts, inner, shared, out, shared_weight=None):
         n_tokens = gate_up.shape[0]
         x = gate_up.to(self.work)
         out.zero_()
@@ -455,7 +531,10 @@ class PlainOps:
         out[:, :n_experts * inner] = (factor[:, :, None] * (g * torch.sigmoid(g) * u)).reshape(n_tokens, -1).to(out.dtype)
         if shared:
             g, u = x[:, n_experts * 2 * inner:n_experts * 2 * inner + shared], x[:, n_experts * 2 * inner + shared:]
-            out[:, n_experts * inner:n_experts * inner + shared] = (g * torch.sigmoid(g) * u).to(out.dtype)
+            both = g * torch.sigmoid(g) * u
+            if shared_weight is not None:
+                both = both * shared_weight.to(self.work)[:, None]
+            out[:, n_experts * inner:n_experts * inner + shared] = both.to(out.dtype)
         return out
 
     def linear(self, x, weight, bias=None, out=None, out_dtype=None):

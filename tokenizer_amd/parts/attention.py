@@ -37,7 +37,8 @@ class GQAttention(Mixer):
     query, at their true positions), `qk_norm` "whole" (an RMS norm with weights `q_norm` [n_heads d] / `k_norm`
     [n_kv d] over all query rows at once and over all key rows at once, before the rotation) and `head_gate`
     (head h's output times sigmoid(W_g x)_h, W_g = `gate_proj.weight` [n_heads, hidden], read from the mixer's
-    input; the gate's rows ride in the joined projection).  For the kernels the maps of differential heads are
+    input; the gate's rows ride in the joined projection) and `softcap` c (a scaled score s becomes c tanh(s / c)
+    before the softmax); `sink` joins these too.  For the kernels the maps of differential heads are
     heads of their own: the query rows are reordered at load time to (kv head, map, head within the group), so
     that map m of kv head g is key head 2 g + m in the ordinary grouping, and key heads 2 g and 2 g + 1 read
     value head g (`value_heads`).
@@ -81,12 +82,16 @@ class GQAttention(Mixer):
     @staticmethod
     def _is_extended(spec: MixerSpec) -> bool:
         return (spec.differential is not None or bool(spec.keep_first) or spec.qk_norm is not None or spec.head_gate
-                or (spec.position is not None and spec.position.kind == "rope_partial"))
+                or spec.softcap is not None or (spec.position is not None and spec.position.kind == "rope_partial"))
 
     def _build_extended(self, spec: MixerSpec, tensors: dict[str, torch.Tensor], runtime: Runtime) -> None:
-        if not spec.own_kv or spec.chunk is not None or spec.distance_bias is not None or spec.sink or spec.out_bias:
-            raise ValueError("differential maps, kept first keys, normalised projections, head gates and the partial "
-                             "rotation do not combine with chunks, distance bias, sinks, borrowed keys or an output bias")
+        if not spec.own_kv or spec.chunk is not None or spec.distance_bias is not None or spec.out_bias:
+            raise ValueError("differential maps, kept first keys, normalised projections, head gates, capped scores and "
+                             "the partial rotation do not combine with chunks, distance bias, borrowed keys or an output bias")
+        if spec.sink and spec.differential is not None:
+            raise ValueError("a sink belongs to one softmax a head, not to the two maps of a differential head")
+        if spec.softcap is not None and not spec.softcap > 0:
+            raise ValueError(f"a cap on the scores is positive, found {spec.softcap}")
         if spec.qk_norm not in (None, "whole"):
             raise ValueError(f"qk_norm {spec.qk_norm!r}: known is \"whole\"")
         H, G, d, dv, hidden = self.n_q, self.n_kv, self.d, self.dv, spec.hidden_size
@@ -121,6 +126,12 @@ class GQAttention(Mixer):
         self.q_norm = by_kv_head(tensors["q_norm"]).to(torch.float32).contiguous() if spec.qk_norm else None
         self.k_norm = tensors["k_norm"].to(torch.float32).contiguous() if spec.qk_norm else None
         self.head_gate, self.eps = spec.head_gate, float(spec.eps)
+        # (A sink and a cap on the scores are handed to the attention kernels only where a layer has them.)
+        self.more = {}
+        if spec.sink:
+            self.more["sinks"] = tensors["sink"].to(torch.float32).contiguous()
+        if spec.softcap is not None:
+            self.more["softcap"] = float(spec.softcap)
         self.w_o, self.b_o = tensors["o_proj.weight"], None
         self.scale = float(spec.scale) if spec.scale is not None else 1.0 / math.sqrt(d)
         self.window = spec.window
@@ -227,7 +238,7 @@ class GQAttention(Mixer):
         ops.paged_attention(qkv, mixed, cache.k_pages, cache.v_pages, ctx.positions, ctx.entry_of_token,
                             ctx.block_tables[cache.group], heads, key_heads, self.d, self.window, self.scale,
                             max_position=ctx.max_position, batch=ctx, value_dim=self.dv, keep_first=self.keep_first,
-                            value_heads=self.n_kv)
+                            value_heads=self.n_kv, **self.more)
         if self.maps > 1:
             out = torch.empty((x.shape[0], self.n_q * self.dv), dtype=x.dtype, device=x.device)
             ops.differential_heads(mixed, self.lam, self.eps, self.out_scale, self.n_q, self.group, self.dv, out)

@@ -229,6 +229,42 @@ class SumDelta:
         return zero
 
 
+class ScaledSum:
+    """What a layer hands on whose sub-layers' outputs are still to be weighted and added: `terms`, each (rows [T, H] in
+    the compute dtype, a factor, a scale float32 [H] or None), standing for x + sum(factor * scale * rows) in float32.
+    A norm of the form x / sqrt(mean(x^2) + eps) * w takes it as its delta and does the additions and the norm in one
+    kernel (`ops.add_terms_rmsnorm`); for anyone else `resolve()` gives the sum as a float32 tensor."""
+    MAX_TERMS = 4
+
+    def __init__(self, ops, terms=()):
+        self.ops, self.terms = ops, tuple(terms)
+
+    @classmethod
+    def of(cls, ops, value) -> "ScaledSum":
+        """A sub-layer's output as a sum: one itself, or a tensor as its one term."""
+        if isinstance(value, cls):
+            return value
+        return cls(ops, () if value is None else ((as_tensor(value), 1.0, None),))
+
+    def scaled_by(self, scale, factor: float = 1.0) -> "ScaledSum":
+        """Every term times `factor` and, coordinate by coordinate, `scale` (float32 [H] or None)."""
+        def both(old):
+            return scale if old is None else old if scale is None else (old * scale).contiguous()
+        return ScaledSum(self.ops, tuple((rows, f * float(factor), both(s)) for rows, f, s in self.terms))
+
+    def plus(self, other: "ScaledSum") -> "ScaledSum":
+        out = ScaledSum(self.ops, self.terms + other.terms)
+        if len(out.terms) > self.MAX_TERMS:
+            raise ValueError(f"a sum of more than {self.MAX_TERMS} terms")
+        return out
+
+    def resolve(self) -> torch.Tensor:
+        rows = self.terms[0][0]
+        zero = torch.zeros(rows.shape, dtype=torch.float32, device=rows.device)
+        self.ops.add_terms_rmsnorm(zero, self.terms, None, 0.0, torch.empty_like(rows))
+        return zero
+
+
 def as_tensor(delta):
     """The delta as a tensor: a product still in parts has them added now."""
     resolve = getattr(delta, "resolve", None)

@@ -3,7 +3,7 @@ from __future__ import annotations
 
 import torch
 
-from .base import BLOCKS, Block, NormedDelta, Repeatable, SumDelta, as_tensor, repeatable_of
+from .base import BLOCKS, Block, NormedDelta, Repeatable, ScaledSum, SumDelta, as_tensor, repeatable_of
 from .spec import TensorSpec
 
 
@@ -58,6 +58,61 @@ class ParallelBlock(Block):
         if self.feed_forward is None:
             return mixed
         return SumDelta(self.mixer.runtime.ops, mixed, self.feed_forward.forward(h, ctx))
+
+
+@BLOCKS.register("parallel_scaled")
+class ScaledParallelBlock(Block):
+    """x + (s1 * mixer(norm1(x)) + s2 * feed_forward(norm2(x))): two norms of the same x, one for each sub-layer, and
+    (option `layer_scale`) a learned scale per coordinate on each output (the block's own tensors `ls1`, `ls2` [width]).
+    The outputs are handed on as the terms of a `ScaledSum`: the next norm weights and adds them to the float32 stream
+    and normalises the sum in one kernel.  Where both norms are of the form x / sqrt(mean(x^2) + eps) * w, that kernel
+    also gives both normalised copies of the row at once.  A mixer may itself hand back a `ScaledSum` (two mixers
+    side by side): its terms join the layer's.  A layer without a feed-forward hands the mixer's terms on alone."""
+    graph_safe = True
+
+    @staticmethod
+    def tensor_specs(layer) -> dict:
+        width, out = int(layer.options["width"]), {}
+        if layer.options.get("layer_scale"):
+            out["ls1"] = TensorSpec((width,), init="ones", role="vector")
+            if layer.feed_forward is not None:
+                out["ls2"] = TensorSpec((width,), init="ones", role="vector")
+        return out
+
+    def __init__(self, mixer_norm, mixer, feed_forward_norm, feed_forward, layer, tensors, runtime):
+        if mixer is None:
+            raise ValueError("a parallel layer has a mixer")
+        self.mixer_norm, self.mixer = mixer_norm, mixer
+        self.feed_forward_norm, self.feed_forward = feed_forward_norm, feed_forward
+        self.runtime = runtime
+        scaled = bool(layer.options.get("layer_scale"))
+        self.mixer_scale = tensors["ls1"].to(torch.float32).contiguous() if scaled else None
+        self.ff_scale = tensors["ls2"].to(torch.float32).contiguous() if scaled and feed_forward is not None else None
+
+    def _normed(self, residual, delta):
+        """Both sub-layers' inputs from the stream and what is still to be added to it."""
+        if self.feed_forward is None:
+            return self.mixer_norm.apply(residual, delta), None
+        ops = self.runtime.ops
+        first, second = self.mixer_norm.fold(), self.feed_forward_norm.fold()
+        if first is not None and second is not None and hasattr(ops, "add_terms_rmsnorm") \
+                and (delta is None or isinstance(delta, (ScaledSum, torch.Tensor))):
+            shape = (residual.shape[0], residual.shape[1])
+            h1 = torch.empty(shape, dtype=self.runtime.dtype, device=residual.device)
+            h2 = torch.empty(shape, dtype=self.runtime.dtype, device=residual.device)
+            ops.add_terms_rmsnorm(residual, ScaledSum.of(ops, delta).terms, first.weight, first.eps, h1,
+                                  weight2=second.weight, eps2=second.eps, out2=h2)
+            return h1, h2
+        h1 = self.mixer_norm.apply(residual, delta)
+        return h1, self.feed_forward_norm.apply(residual, None)
+
+    def forward(self, residual, delta, ctx, cache):
+        ops = self.runtime.ops
+        h1, h2 = self._normed(residual, delta)
+        out = ScaledSum.of(ops, self.mixer.forward(h1, ctx, cache)).scaled_by(self.mixer_scale)
+        if self.feed_forward is not None:
+            out = out.plus(ScaledSum.of(ops, self.feed_forward.forward(h2, ctx)).scaled_by(self.ff_scale))
+        return out
 
 
 @BLOCKS.register("sandwich_norm")

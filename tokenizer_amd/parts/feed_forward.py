@@ -86,6 +86,38 @@ class GatedDense(FeedForward):
         return ops.linear(act, self.w_down, pending=True) if pending else ops.linear(act, self.w_down)
 
 
+@FEED_FORWARDS.register("plain_dense")
+class PlainDense(FeedForward):
+    """down(act(up(x))) without a gate branch and without biases; `activation` "relu2" is max(z, 0)^2 (computed in
+    float32 from what the first product leaves).  Tensors `up` [inner, hidden], `down` [hidden, inner]."""
+    graph_safe = True
+
+    def __init__(self, spec: FeedForwardSpec, tensors: dict[str, torch.Tensor], runtime: Runtime):
+        if spec.activation != "relu2":
+            raise ValueError(f"plain_dense knows the activation relu2, not {spec.activation!r}")
+        self.spec, self.runtime = spec, runtime
+        up, down = tensors["up"], tensors["down"]
+        # (The bfloat16 products read K in eights: an inner width that is no multiple of eight is filled up with zero
+        # rows of up and zero columns of down.)
+        fill = (-spec.intermediate_size) % 8 if runtime.dtype == torch.bfloat16 else 0
+        if fill:
+            up = torch.cat([up, up.new_zeros((fill, up.shape[1]))], dim=0).contiguous()
+            down = torch.cat([down, down.new_zeros((down.shape[0], fill))], dim=1).contiguous()
+        self.w_up, self.w_down = up, down
+
+    @staticmethod
+    def tensor_specs(spec: FeedForwardSpec) -> dict[str, TensorSpec]:
+        return {"up": TensorSpec((spec.intermediate_size, spec.hidden_size)),
+                "down": TensorSpec((spec.hidden_size, spec.intermediate_size))}
+
+    def forward(self, x, ctx):
+        ops = self.runtime.ops
+        up = ops.linear(x, self.w_up)
+        act = torch.empty_like(up)
+        ops.relu2(up, act)
+        return ops.linear(act, self.w_down)
+
+
 @FEED_FORWARDS.register("routed_experts")
 class RoutedExperts(FeedForward):
     """A mixture of `n_experts` small gated feed-forwards (tensors `e<j>.gate|up|down`, inner width
@@ -110,7 +142,10 @@ class RoutedExperts(FeedForward):
     (a tensor, one number an expert); with `n_groups` the experts form that many equal groups of neighbours, a group is
     worth the sum of its two largest choice scores, and only experts of the `keep_groups` best groups can be chosen
     (the others count as minus infinity); the `top_k` largest choice scores are chosen and weighted by their s over
-    the chosen's sum (+ 1e-20).  Logits, scores and weights are float32.
+    the chosen's sum (+ 1e-20).  `router` "softmax_all": the same with s = softmax over all experts and no correction;
+    `group_worth` "max": a group is worth its largest choice score.  `shared_gate`: the shared expert's output times
+    sigmoid(W_sg x), one number a token (tensor `shared.sg` [1, hidden]; its row rides behind the router's rows, so
+    the gate's logit is a float32 sum of the same product).  Logits, scores and weights are float32.
     """
     graph_safe = True
     GROUPED_FROM = 1024        # (token, expert) pairs from which the sorted form runs
@@ -121,17 +156,25 @@ class RoutedExperts(FeedForward):
                              f"{'gated' if spec.gated else 'ungated'} {spec.activation!r}")
         if not 0 < spec.top_k <= spec.n_experts:
             raise ValueError(f"{spec.top_k} of {spec.n_experts} experts")
-        if spec.router not in ("softmax", "sigmoid"):
-            raise ValueError(f"router {spec.router!r}: known are softmax and sigmoid")
+        if spec.router not in ("softmax", "sigmoid", "softmax_all"):
+            raise ValueError(f"router {spec.router!r}: known are softmax, sigmoid and softmax_all")
+        if spec.group_worth not in ("top2", "max"):
+            raise ValueError(f"group_worth {spec.group_worth!r}: known are top2 and max")
         self.spec, self.runtime = spec, runtime
         self.n_experts, self.top_k = spec.n_experts, spec.top_k
         self.inner, self.shared = spec.intermediate_size, spec.shared_size
         self.gated, self.sigmoid = spec.gated, spec.router == "sigmoid"
+        self.scored = spec.router in ("sigmoid", "softmax_all")      # chosen by scores, weighted by them over their sum
         if not self.gated and self.shared:
             raise ValueError("ungated experts have no shared expert here")
+        self.shared_gate = bool(spec.shared_gate) and bool(self.shared)
+        if self.shared_gate and not self.scored:
+            raise ValueError("the shared expert's gate rides in the scored routers' logits")
         self.w_router = tensors["router"]
-        if self.sigmoid:
-            self.correction = tensors["correction"].to(torch.float32).contiguous()
+        if self.shared_gate:          # the gate's row behind the experts' rows: its logit comes out of the same product
+            self.w_router = torch.cat([self.w_router, tensors["shared.sg"].reshape(1, -1)], dim=0).contiguous()
+        if self.scored:
+            self.correction = tensors["correction"].to(torch.float32).contiguous() if self.sigmoid else None
             self.n_groups, self.keep_groups = int(spec.n_groups), int(spec.keep_groups)
             if self.n_groups and (self.n_experts % self.n_groups or not 0 < self.keep_groups <= self.n_groups
                                   or self.keep_groups * (self.n_experts // self.n_groups) < self.top_k):
@@ -161,6 +204,8 @@ class RoutedExperts(FeedForward):
         out = {"router": TensorSpec((spec.n_experts, spec.hidden_size), std=0.5)}
         if spec.router == "sigmoid":
             out["correction"] = TensorSpec((spec.n_experts,), role="vector", std=0.2)
+        if spec.shared_gate and spec.shared_size:
+            out["shared.sg"] = TensorSpec((1, spec.hidden_size), std=0.5)
         sizes = [(f"e{j}", spec.intermediate_size) for j in range(spec.n_experts)]
         if spec.shared_size:
             sizes.append(("shared", spec.shared_size))
@@ -174,27 +219,36 @@ class RoutedExperts(FeedForward):
         ops = self.runtime.ops
         chosen = torch.empty((x.shape[0], self.top_k), dtype=torch.int32, device=x.device)
         weights = torch.empty((x.shape[0], self.top_k), dtype=torch.float32, device=x.device)
-        if self.sigmoid:
+        shared_weight = None
+        if self.sigmoid and not self.shared_gate and self.spec.group_worth == "top2":
             fused = getattr(ops, "route_rows_sigmoid", None)   # few rows: the router's product and the choice in one kernel
             if (fused is None or x.shape[0] > ops.ROUTE_ROWS_FUSED
                     or not fused(x, self.w_router, self.correction, self.n_groups, self.keep_groups, chosen, weights)):
                 ops.route_sigmoid(ops.linear(x, self.w_router, out_dtype=torch.float32), self.correction, self.n_groups,
                                   self.keep_groups, chosen, weights)
+        elif self.scored:
+            if self.shared_gate:
+                shared_weight = torch.empty((x.shape[0],), dtype=torch.float32, device=x.device)
+            ops.route_scores(ops.linear(x, self.w_router, out_dtype=torch.float32), self.correction, self.n_experts,
+                             self.n_groups, self.keep_groups, chosen, weights, softmax=not self.sigmoid,
+                             group_max=self.spec.group_worth == "max", gate=shared_weight)
         else:
             fused = getattr(ops, "route_rows", None)      # the router's product and the choice in one kernel, where there is one
             if fused is None or not fused(x, self.w_router, chosen, weights):
                 ops.route_top(ops.linear(x, self.w_router, out_dtype=torch.float32), chosen, weights)
         if self.groupable and x.shape[0] * self.top_k >= self.GROUPED_FROM and hasattr(ops, "grouped_linear"):
-            return self._sorted(x, chosen, weights)
+            return self._sorted(x, chosen, weights, shared_weight)
         gate_up = ops.linear(x, self.w_gate_up)
         act = torch.empty((x.shape[0], self.columns), dtype=x.dtype, device=x.device)
-        if self.gated:
+        if self.gated and shared_weight is not None:
+            ops.expert_gate(gate_up, chosen, weights, self.n_experts, self.inner, self.shared, act, shared_weight=shared_weight)
+        elif self.gated:
             ops.expert_gate(gate_up, chosen, weights, self.n_experts, self.inner, self.shared, act)
         else:
             ops.expert_act(gate_up, chosen, weights, self.n_experts, self.inner, act)
         return ops.linear(act, self.w_down)
 
-    def _sorted(self, x, chosen, weights):
+    def _sorted(self, x, chosen, weights, shared_weight=None):
         """Tiles of rows that belong to one expert each: gate/up, the activation, down, then a token's experts added up."""
         ops = self.runtime.ops
         hidden, inner = x.shape[1], self.inner
@@ -212,4 +266,6 @@ class RoutedExperts(FeedForward):
         if self.shared:
             shared = ops.linear(ops.linear_silu_gate(x, self.w_shared_gate_up), self.w_shared_down)
         out = torch.empty((x.shape[0], hidden), dtype=x.dtype, device=x.device)
+        if shared_weight is not None:
+            return ops.expert_combine(rows, slot_of, weights, shared, out, shared_weight=shared_weight)
         return ops.expert_combine(rows, slot_of, weights, shared, out)

@@ -5,7 +5,7 @@ import dataclasses
 
 import torch
 
-from .base import BLOCKS, FEED_FORWARDS, FRAMES, MIXERS, NORMS, Runtime, repeatable_of
+from .base import BLOCKS, FEED_FORWARDS, FRAMES, MIXERS, NORMS, Runtime, ScaledSum, repeatable_of
 from .spec import CacheNeed, ModelSpec, TensorSpec
 
 
@@ -169,6 +169,9 @@ class DecoderModel:
         out.update(_prefixed(spec.final_norm_prefix, NORMS.get(spec.final_norm.kind).tensor_specs(spec.final_norm)))
         if not spec.tied_head:
             out[spec.head_name] = TensorSpec((spec.vocab_size, spec.hidden_size))
+        pass_input = spec.options.get("pass_input")
+        if pass_input:
+            out[pass_input["tensor"]] = TensorSpec((spec.hidden_size, 2 * spec.hidden_size))
         return out
 
     @staticmethod
@@ -205,6 +208,15 @@ class DecoderModel:
                                          runtime=runtime))
             else:
                 self.blocks.append(block(mixer_norm, mixer, ff_norm, feed_forward))
+        # Options of the frame.  `pass_input` {"tensor": name, "before": schedule indices}: in front of those scheduled
+        # layers the stream x becomes W [x; x0] with W [hidden, 2 hidden] and x0 the embedding's output (a run of
+        # layers that is gone through several times takes the token in again at the start of every pass).
+        # `logit_scale` s and `logit_cap` c: the logits are c tanh(s z / c).
+        pass_input = spec.options.get("pass_input") or {}
+        self.pass_before = frozenset(int(index) for index in pass_input.get("before", ()))
+        self.pass_weight = tensors[pass_input["tensor"]] if self.pass_before else None
+        self.logit_scale = float(spec.options.get("logit_scale") or 1.0)
+        self.logit_cap = float(spec.options.get("logit_cap") or 0.0)
         self.final_norm = NORMS.get(spec.final_norm.kind)(spec.final_norm, _strip(spec.final_norm_prefix, tensors), runtime)
         self.head = self.embedding if spec.tied_head else tensors[spec.head_name]
         parts = [self.final_norm] + [p for b in self.blocks if hasattr(b, "mixer")
@@ -239,20 +251,37 @@ class DecoderModel:
         rows are normalised and multiplied with the head (the reference keeps the last row,
         qwen-infer/src/model.rs:1224-1242)."""
         wanted = self.final_norm.apply(residual, delta, rows=ctx.want_rows)
-        return self.runtime.ops.linear(wanted, self.head, out_dtype=torch.float32)
+        logits = self.runtime.ops.linear(wanted, self.head, out_dtype=torch.float32)
+        if self.logit_scale != 1.0 or self.logit_cap:
+            self.runtime.ops.scale_cap(logits, self.logit_scale, self.logit_cap)
+        return logits
+
+    def take_in_again(self, residual: torch.Tensor, delta, both: torch.Tensor) -> torch.Tensor:
+        """The stream behind a pass's input: `both` [tokens, 2 hidden] (compute dtype) holds the embedding's output in
+        its right half; the stream with everything still to be added goes into the left half, and the product with
+        the pass's matrix, a float32 sum, is the new stream."""
+        ops, hidden = self.runtime.ops, self.spec.hidden_size
+        ops.add_terms_rmsnorm(residual, ScaledSum.of(ops, delta).terms, None, 0.0, both[:, :hidden], store_residual=False)
+        return ops.linear(both, self.pass_weight, out_dtype=torch.float32)
 
     def forward(self, ctx, layer_caches: list[LayerCache]) -> torch.Tensor:
         """Run the tokens of `ctx` through the schedule; float32 logits [len(want_rows), vocab]."""
         ops = self.runtime.ops
         residual = self.embed(ctx)
         delta = None
+        both = None
+        if self.pass_before:                       # the embedding's output is kept, in the right half of a row of two
+            both = torch.empty((ctx.n_tokens, 2 * self.spec.hidden_size), dtype=self.runtime.dtype, device=self.runtime.device)
+            ops.add_terms_rmsnorm(residual, (), None, 0.0, both[:, self.spec.hidden_size:], store_residual=False)
         # Like layers make the same library calls on a batch: the calls of the first are recorded and made again
         # for the others with their tensors' addresses put in place, which spares those layers' Python (about
         # two thirds of an eager step's host time; a step of a small model is bound by it).  Not while a graph
         # is recorded or warmed up: that happens once, and the library times its products there.
         record = getattr(ops, "record_launches", None) if self.repeat_layers and not getattr(ops, "capturing", False) else None
         tapes: dict = {}
-        for entry, cache in zip(self.spec.schedule, layer_caches):
+        for at, (entry, cache) in enumerate(zip(self.spec.schedule, layer_caches)):
+            if at in self.pass_before:
+                residual, delta = self.take_in_again(residual, delta, both), None
             block = self.blocks[entry.layer]
             make = self._make_of(block, entry.layer, cache) if record is not None else None
             form, addresses = _coming(delta) if make is not None else (None, ())

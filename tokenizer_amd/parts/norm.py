@@ -3,7 +3,7 @@ from __future__ import annotations
 
 import torch
 
-from .base import NORMS, Norm, NormedDelta, NormFold, Repeatable, Runtime, SumDelta
+from .base import NORMS, Norm, NormedDelta, NormFold, Repeatable, Runtime, ScaledSum, SumDelta
 from .spec import NormSpec, TensorSpec
 
 
@@ -14,7 +14,7 @@ class RMSNorm(Norm):
     tensor that the prefix itself names.  Option `offset` c: the stored tensor lies around zero and the scale is
     c + weight (formed once, in float32).  A delta that is itself still to be normalised (`NormedDelta`) is
     normalised, scaled and added in the same kernel; so are the two terms of a `SumDelta` (two sub-layers that read
-    the same normalised rows)."""
+    the same normalised rows) and the weighted terms of a `ScaledSum`."""
     graph_safe = True
 
 
@@ -44,6 +44,9 @@ class RMSNorm(Norm):
         if isinstance(delta, SumDelta):
             return self.runtime.ops.add_pair_rmsnorm(residual, delta.first, delta.second, self.weight, self.eps, out, rows,
                                                      store_residual=rows is None)
+        if isinstance(delta, ScaledSum):
+            return self.runtime.ops.add_terms_rmsnorm(residual, delta.terms, self.weight, self.eps, out, rows,
+                                                      store_residual=rows is None)
         if isinstance(delta, NormedDelta):
             if delta.side is not None:
                 done = delta.side.fused(residual, delta, self.weight, self.eps, out, rows)

@@ -127,6 +127,10 @@ class MixerSpec:
     #                               one rotated key part shared by all heads (0: no positions at all)
     element_gate: bool = False    # the mixer's output times sigmoid of a projection of its input, coordinate by coordinate
     conv_taps: int = 0            # recurrent mixers: taps of the short causal convolution over q, k and v (0: none)
+    softcap: float | None = None  # c: a score (scaled, biased) becomes c tanh(score / c) before the softmax
+    inner_size: int = 0           # selective scan: channels of the recurrence
+    state_dim: int = 0            # selective scan: numbers of state a channel keeps
+    dt_rank: int = 0              # selective scan: width of the narrow projection the step sizes are made from
     tensor_names: tuple[tuple[str, str], ...] = ()   # (part's name, file's name) where a file names tensors otherwise
     options: dict[str, Any] = dataclasses.field(default_factory=dict, hash=False, compare=False)
 
@@ -146,10 +150,14 @@ class FeedForwardSpec:
     gated: bool = True            # experts are down(act(gate) * up); False: down(act(up)), tensors `up` and `down` alone
     router: str = "softmax"       # "softmax": the largest logits, weighted by the softmax over the chosen; "sigmoid":
     #                               scores s = sigmoid(logit), chosen by s + `correction` (a tensor, one number an
-    #                               expert), weighted by s over the chosen's sum
+    #                               expert), weighted by s over the chosen's sum; "softmax_all": scores s = softmax
+    #                               over all experts, chosen by s, weighted by s over the chosen's sum
     n_groups: int = 0             # "sigmoid": experts form so many equal groups of neighbours (0: no groups) ...
     keep_groups: int = 0          # ... of which only the best so many (by the sum of a group's two largest choice
     #                               scores) can be chosen from
+    group_worth: str = "top2"     # what a group is worth: "top2" (the sum of its two largest choice scores) or "max"
+    shared_gate: bool = False     # the shared expert's output times sigmoid of one number projected from the input
+    #                               (tensor `shared.sg` [1, hidden])
     tensor_names: tuple[tuple[str, str], ...] = ()
     options: dict[str, Any] = dataclasses.field(default_factory=dict, hash=False, compare=False)
 
