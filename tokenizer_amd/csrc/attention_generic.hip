@@ -15,6 +15,7 @@
 // sinks (float [n_q] or null): exp(sinks[h]) joins the softmax's denominator (no key, no value, not scaled, no bias).
 // keep_first > 0 (with a window): keys at positions below keep_first stay visible behind the window, at their own positions.
 // n_v (a divisor of n_kv): the value pages hold n_v heads, and key head g reads value head g / (n_kv / n_v).
+// softcap > 0: a score s (scaled, with its distance term) becomes softcap * tanh(s / softcap) before the softmax.
 template <typename T>
 __global__ void __launch_bounds__(ATT_WAVES * WAVE)
 paged_attention_generic(const T* __restrict__ q, int q_stride, T* __restrict__ out,
@@ -22,7 +23,8 @@ paged_attention_generic(const T* __restrict__ q, int q_stride, T* __restrict__ o
                         const int* __restrict__ positions, const int* __restrict__ entry_of_token,
                         const int* __restrict__ block_table, int table_stride,
                         int n_q, int n_kv, int d, int page_size, int window, float scale, int dv, int chunk,
-                        const float* __restrict__ slopes, const float* __restrict__ sinks, int keep_first, int n_v) {
+                        const float* __restrict__ slopes, const float* __restrict__ sinks, int keep_first, int n_v,
+                        float softcap) {
   __shared__ float q_s[ATT_MAX_D];
   __shared__ float acc_s[ATT_WAVES][ATT_MAX_D];
   __shared__ float m_s[ATT_WAVES], l_s[ATT_WAVES];
@@ -70,6 +72,7 @@ paged_attention_generic(const T* __restrict__ q, int q_stride, T* __restrict__ o
         for (int i = 0; i < d; ++i) dot += q_s[i] * ld(kr + i);
       }
       s = dot * scale - slope * (float)(pos - j);
+      if (softcap > 0.f) s = softcap * tanhf(s / softcap);
     }
     const float m_new = fmaxf(m, wave_max(s));
     const float p = valid ? expf(s - m_new) : 0.f;
@@ -159,7 +162,7 @@ extern "C" int ta_paged_attention_generic(const void* q, int q_stride, void* out
                                           const void* block_table, int table_stride, int n_tokens, int n_q,
                                           int n_kv, int d, int page_size, int window, float scale, int dtype,
                                           int dv, int chunk, const void* slopes, const void* sinks,
-                                          int keep_first, int n_v, hipStream_t stream) {
+                                          int keep_first, int n_v, float softcap, hipStream_t stream) {
   if (n_tokens <= 0) return 0;
   if (dv <= 0) dv = d;
   if (n_v <= 0) n_v = n_kv;
@@ -169,11 +172,11 @@ extern "C" int ta_paged_attention_generic(const void* q, int q_stride, void* out
     paged_attention_generic<float><<<grid, ATT_WAVES * WAVE, 0, stream>>>((const float*)q, q_stride, (float*)out,
         (const float*)k_pages, (const float*)v_pages, (const int*)positions, (const int*)entry_of_token,
         (const int*)block_table, table_stride, n_q, n_kv, d, page_size, window, scale, dv, chunk,
-        (const float*)slopes, (const float*)sinks, keep_first, n_v);
+        (const float*)slopes, (const float*)sinks, keep_first, n_v, softcap);
   else
     paged_attention_generic<bf16_t><<<grid, ATT_WAVES * WAVE, 0, stream>>>((const bf16_t*)q, q_stride, (bf16_t*)out,
         (const bf16_t*)k_pages, (const bf16_t*)v_pages, (const int*)positions, (const int*)entry_of_token,
         (const int*)block_table, table_stride, n_q, n_kv, d, page_size, window, scale, dv, chunk,
-        (const float*)slopes, (const float*)sinks, keep_first, n_v);
+        (const float*)slopes, (const float*)sinks, keep_first, n_v, softcap);
   return LAUNCH_STATUS();
 }

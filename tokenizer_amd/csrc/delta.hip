@@ -32,7 +32,7 @@ __device__ __forceinline__ int conv_column(const ConvRuns& runs, int c) {
   return runs.offset[2] + c - runs.width[1];
 }
 
-// out[t, c] = silu(sum_j taps[c, j] * x[t - (n_taps - 1) + j, c]): inputs before the portion's first row come from the
+// out[t, c] = silu(bias[c] + sum_j taps[c, j] * x[t - (n_taps - 1) + j, c]) (bias float [channels], or null): inputs before the portion's first row come from the
 // entry's state row (its last n_taps - 1 inputs, oldest first), and are zeros if the portion starts at position 0.
 // A thread a (token, channel); blockIdx.x is the token.
 template <typename T>
@@ -40,7 +40,8 @@ __global__ void __launch_bounds__(256)
 short_conv_silu_kernel(const T* __restrict__ rows, int row_stride, ConvRuns runs, int channels, const float* __restrict__ taps,
                        int n_taps, const float* __restrict__ state, size_t state_stride, int state_offset,
                        const int* __restrict__ cu_q, const int* __restrict__ first_position,
-                       const int* __restrict__ state_slots, const int* __restrict__ entry_of_token, T* __restrict__ out) {
+                       const int* __restrict__ state_slots, const int* __restrict__ entry_of_token, T* __restrict__ out,
+                       const float* __restrict__ bias) {
   const int t = blockIdx.x, c = blockIdx.y * 256 + threadIdx.x;
   if (c >= channels) return;
   const int e = entry_of_token[t];
@@ -52,7 +53,7 @@ short_conv_silu_kernel(const T* __restrict__ rows, int row_stride, ConvRuns runs
   const bool zeros = first_position[e] == 0;
   const float* tail = state + (size_t)state_slots[e] * state_stride + state_offset;
   const int column = conv_column(runs, c);
-  float y = 0.f;
+  float y = bias ? bias[c] : 0.f;
   for (int j = 0; j < n_taps; ++j) {
     const int src = t - (n_taps - 1) + j;
     float x;
@@ -282,7 +283,7 @@ extern "C" int ta_short_conv_silu(const void* rows, int row_stride, int o0, int 
                                   const void* taps, int n_taps, void* state, long state_stride, int state_offset,
                                   const void* cu_q, const void* first_position, const void* state_slots,
                                   const void* entry_of_token, void* out, int n_tokens, int n_entries, int dtype,
-                                  hipStream_t stream) {
+                                  const void* bias, hipStream_t stream) {
   if (n_tokens <= 0 || n_entries <= 0) return 0;
   const int channels = w0 + w1 + w2;
   if (channels <= 0 || w0 < 0 || w1 < 0 || w2 < 0 || n_taps < 1 || n_taps > DL_MAX_TAPS || channels > 65535 * 256 ||
@@ -293,7 +294,7 @@ extern "C" int ta_short_conv_silu(const void* rows, int row_stride, int o0, int 
 #define CONV(TT)                                                                                                           \
   short_conv_silu_kernel<TT><<<per_token, 256, 0, stream>>>((const TT*)rows, row_stride, runs, channels, (const float*)taps, \
       n_taps, (const float*)state, (size_t)state_stride, state_offset, (const int*)cu_q, (const int*)first_position,        \
-      (const int*)state_slots, (const int*)entry_of_token, (TT*)out);                                                      \
+      (const int*)state_slots, (const int*)entry_of_token, (TT*)out, (const float*)bias);                                  \
   if (n_taps > 1)                                                                                                          \
     short_conv_keep_kernel<TT><<<per_entry, 256, 0, stream>>>((const TT*)rows, row_stride, runs, channels, n_taps,          \
         (float*)state, (size_t)state_stride, state_offset, (const int*)cu_q, (const int*)first_position,                   \

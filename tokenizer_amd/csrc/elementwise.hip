@@ -330,6 +330,104 @@ extern "C" int ta_add_pair_rmsnorm(void* residual, const void* first, const void
   return LAUNCH_STATUS();
 }
 
+// Sub-layers' outputs still to be weighted and added: up to four terms, term k = factor[k] * scale[k][h] * rows[k][r, h]
+// (scale float [hidden] or null).  For output row i, r = rows ? rows[i] : i; x = residual[r] + (the terms' sum), all
+// float; if store_residual: residual[r] = x; out[i] = weight ? x / sqrt(mean(x^2) + eps) * weight : x, in rows of
+// `out_stride` elements; with out2, a second normalised copy under weight2 and eps2.  A row a workgroup; the row is
+// read once and kept in registers.
+#define TERMS_MAX 4
+struct SumTerms {
+  const void* rows[TERMS_MAX];
+  const float* scale[TERMS_MAX];
+  float factor[TERMS_MAX];
+  int count;
+};
+
+template <typename T, int PER>
+__global__ void __launch_bounds__(256)
+add_terms_rmsnorm_kernel(float* __restrict__ residual, SumTerms terms, const float* __restrict__ weight, float eps,
+                         T* __restrict__ out, int out_stride, const float* __restrict__ weight2, float eps2,
+                         T* __restrict__ out2, const int* __restrict__ rows, int hidden, int store_residual) {
+  __shared__ float scratch[16];
+  const int i = blockIdx.x;
+  const int r = rows ? rows[i] : i;
+  float* res = residual + (size_t)r * hidden;
+  float x[PER];
+  float sq = 0.f;
+#pragma unroll
+  for (int p = 0; p < PER; ++p) {
+    const int h = p * 256 + threadIdx.x;
+    x[p] = 0.f;
+    if (h < hidden) {
+      float sum = 0.f;
+#pragma unroll
+      for (int k = 0; k < TERMS_MAX; ++k)
+        if (k < terms.count) {
+          float v = terms.factor[k] * ld(reinterpret_cast<const T*>(terms.rows[k]) + (size_t)r * hidden + h);
+          if (terms.scale[k]) v *= terms.scale[k][h];
+          sum = k == 0 ? v : sum + v;
+        }
+      x[p] = terms.count > 0 ? res[h] + sum : res[h];
+      if (store_residual) res[h] = x[p];
+    }
+    sq += x[p] * x[p];
+  }
+  float mean = 0.f;
+  if (weight || out2) mean = block_sum(sq, scratch) / (float)hidden;
+  const float inv = weight ? 1.0f / sqrtf(mean + eps) : 1.f;
+  T* dst = out + (size_t)i * out_stride;
+#pragma unroll
+  for (int p = 0; p < PER; ++p) {
+    const int h = p * 256 + threadIdx.x;
+    if (h < hidden) st(dst + h, weight ? x[p] * inv * weight[h] : x[p]);
+  }
+  if (out2) {
+    const float inv2 = 1.0f / sqrtf(mean + eps2);
+    T* dst2 = out2 + (size_t)i * hidden;
+#pragma unroll
+    for (int p = 0; p < PER; ++p) {
+      const int h = p * 256 + threadIdx.x;
+      if (h < hidden) st(dst2 + h, x[p] * inv2 * weight2[h]);
+    }
+  }
+}
+
+extern "C" int ta_add_terms_rmsnorm(void* residual, int count, const void* rows0, const void* rows1, const void* rows2,
+                                    const void* rows3, const void* scale0, const void* scale1, const void* scale2,
+                                    const void* scale3, float f0, float f1, float f2, float f3, const void* weight,
+                                    float eps, void* out, int out_stride, const void* weight2, float eps2, void* out2,
+                                    const void* rows, int n_rows, int hidden, int store_residual, int dtype,
+                                    hipStream_t stream) {
+  if (n_rows <= 0) return 0;
+  if (hidden <= 0 || hidden > 256 * 32 || count < 0 || count > TERMS_MAX || out_stride < hidden || (out2 && !weight2)) return -1;
+  SumTerms terms = {{rows0, rows1, rows2, rows3},
+                    {(const float*)scale0, (const float*)scale1, (const float*)scale2, (const float*)scale3},
+                    {f0, f1, f2, f3}, count};
+  for (int k = 0; k < count; ++k)
+    if (!terms.rows[k]) return -1;
+#define TERMS(TT, PP) add_terms_rmsnorm_kernel<TT, PP><<<n_rows, 256, 0, stream>>>((float*)residual, terms,     (const float*)weight, eps, (TT*)out, out_stride, (const float*)weight2, eps2, (TT*)out2, (const int*)rows, hidden, store_residual)
+#define TERMS_SIZES(TT) if (hidden <= 256) TERMS(TT, 1); else if (hidden <= 1024) TERMS(TT, 4); else if (hidden <= 2048) TERMS(TT, 8);                         else if (hidden <= 4096) TERMS(TT, 16); else TERMS(TT, 32)
+  if (dtype == DT_F32) { TERMS_SIZES(float); } else { TERMS_SIZES(bf16_t); }
+#undef TERMS_SIZES
+#undef TERMS
+  return LAUNCH_STATUS();
+}
+
+// x <- cap > 0 ? cap * tanh(scale * x / cap) : scale * x, in place, float.
+__global__ void scale_cap_kernel(float* __restrict__ x, size_t total, float scale, float cap) {
+  for (size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += (size_t)gridDim.x * blockDim.x) {
+    const float v = x[idx] * scale;
+    x[idx] = cap > 0.f ? cap * tanhf(v / cap) : v;
+  }
+}
+
+extern "C" int ta_scale_cap(void* x, size_t total, float scale, float cap, hipStream_t stream) {
+  if (total == 0) return 0;
+  const int blocks = (int)((total + 255) / 256 < 65535 ? (total + 255) / 256 : 65535);
+  scale_cap_kernel<<<blocks, 256, 0, stream>>>((float*)x, total, scale, cap);
+  return LAUNCH_STATUS();
+}
+
 extern "C" int ta_add_rmsnorm(void* residual, const void* delta, const void* weight, void* out,
                               const void* rows, int n_rows, int hidden, float eps, int store_residual,
                               int dtype, hipStream_t stream) {

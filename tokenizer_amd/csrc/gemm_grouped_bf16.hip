@@ -162,16 +162,18 @@ grouped_gemm_bf16_kernel(const bf16_t* __restrict__ A, int lda, const int* __res
     }
 }
 
-// out[t, :] = shared[t, :] (if given) + sum over the token's picks k of weights[t, k] * rows[slot_of[t * top + k], :]
+// out[t, :] = shared[t, :] (if given; times shared_weight[t], float, if that is given) + sum over the token's picks k of weights[t, k] * rows[slot_of[t * top + k], :]
 // (a pick without a slot is passed over).  rows float [*, hidden]; shared and out of type T.
 template <typename T>
 __global__ void expert_combine_kernel(const float* __restrict__ rows, const int* __restrict__ slot_of,
                                       const float* __restrict__ weights, int top, const T* __restrict__ shared,
-                                      T* __restrict__ out, int hidden, size_t total) {
+                                      T* __restrict__ out, int hidden, size_t total,
+                                      const float* __restrict__ shared_weight) {
   for (size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += (size_t)gridDim.x * blockDim.x) {
     const size_t t = idx / hidden;
     const int h = (int)(idx - t * hidden);
     float sum = shared ? ld(shared + idx) : 0.f;
+    if (shared && shared_weight) sum *= shared_weight[t];
     for (int k = 0; k < top; ++k) {
       const int slot = slot_of[t * top + k];
       if (slot >= 0) sum = fmaf(weights[t * top + k], rows[(size_t)slot * hidden + h], sum);
@@ -208,15 +210,18 @@ extern "C" int ta_grouped_gemm_bf16(const void* A, int lda, const void* row_of, 
 }
 
 extern "C" int ta_expert_combine(const void* rows, const void* slot_of, const void* weights, int n_tokens, int top,
-                                 const void* shared, void* out, int hidden, int dtype, hipStream_t stream) {
+                                 const void* shared, void* out, int hidden, int dtype, const void* shared_weight,
+                                 hipStream_t stream) {
   const size_t total = (size_t)n_tokens * hidden;
   if (total == 0) return 0;
   const int blocks = (int)((total + 255) / 256 < 65535 ? (total + 255) / 256 : 65535);
   if (dtype == DT_F32)
     expert_combine_kernel<float><<<blocks, 256, 0, stream>>>((const float*)rows, (const int*)slot_of, (const float*)weights,
-                                                             top, (const float*)shared, (float*)out, hidden, total);
+                                                             top, (const float*)shared, (float*)out, hidden, total,
+                                                             (const float*)shared_weight);
   else
     expert_combine_kernel<bf16_t><<<blocks, 256, 0, stream>>>((const float*)rows, (const int*)slot_of, (const float*)weights,
-                                                              top, (const bf16_t*)shared, (bf16_t*)out, hidden, total);
+                                                              top, (const bf16_t*)shared, (bf16_t*)out, hidden, total,
+                                                              (const float*)shared_weight);
   return LAUNCH_STATUS();
 }

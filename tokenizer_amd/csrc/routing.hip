@@ -143,11 +143,11 @@ route_rows_kernel(const T* __restrict__ x, int lda, const T* __restrict__ router
 // gate_up: [n_tokens, n_experts * 2 * inner + 2 * shared], expert e's gate rows then its up rows, the shared expert
 // last.  out: [n_tokens, columns] with columns >= n_experts * inner + shared: out[t, e * inner + i] =
 // w * silu(gate) * up for an expert the token chose with weight w, 0 for the others; the shared expert's columns
-// with weight 1; columns beyond are 0.
+// with weight 1 (or shared_weight[t], float, where given); columns beyond are 0.
 template <typename T>
 __global__ void expert_gate_kernel(const T* __restrict__ gate_up, const int* __restrict__ chosen,
                                    const float* __restrict__ weights, int top, int n_experts, int inner, int shared,
-                                   int columns, T* __restrict__ out, size_t total) {
+                                   int columns, T* __restrict__ out, size_t total, const float* __restrict__ shared_weight) {
   const int in_stride = n_experts * 2 * inner + 2 * shared;
   for (size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += (size_t)gridDim.x * blockDim.x) {
     const size_t t = idx / columns;
@@ -167,6 +167,7 @@ __global__ void expert_gate_kernel(const T* __restrict__ gate_up, const int* __r
       const int i = c - n_experts * inner;
       const float g = ld(row + (size_t)n_experts * 2 * inner + i), u = ld(row + (size_t)n_experts * 2 * inner + shared + i);
       value = g / (1.0f + expf(-g)) * u;
+      if (shared_weight) value *= shared_weight[t];
     }
     st(out + idx, value);
   }
@@ -201,7 +202,8 @@ __global__ void gelu_gate_kernel(const T* __restrict__ in, T* __restrict__ out, 
 // one expert; the rows of experts a token did not choose are not read.
 __global__ void expert_gate_vec_kernel(const bf16_t* __restrict__ gate_up, const int* __restrict__ chosen,
                                        const float* __restrict__ weights, int top, int n_experts, int inner, int shared,
-                                       int columns, bf16_t* __restrict__ out, size_t total8) {
+                                       int columns, bf16_t* __restrict__ out, size_t total8,
+                                       const float* __restrict__ shared_weight) {
   const int in_stride = n_experts * 2 * inner + 2 * shared, columns8 = columns / 8;
   for (size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total8; idx += (size_t)gridDim.x * blockDim.x) {
     const size_t t = idx / columns8;
@@ -218,7 +220,7 @@ __global__ void expert_gate_vec_kernel(const bf16_t* __restrict__ gate_up, const
     } else if (c < n_experts * inner + shared) {
       g_at = row + (size_t)n_experts * 2 * inner + (c - n_experts * inner);
       up_off = shared;
-      w = 1.f;
+      w = shared_weight ? shared_weight[t] : 1.f;
     }
     uint4 packed = make_uint4(0, 0, 0, 0);
     if (g_at) {
@@ -277,22 +279,23 @@ extern "C" int ta_route_rows(const void* x, int lda, const void* router, int n_t
 }
 
 extern "C" int ta_expert_gate(const void* gate_up, const void* chosen, const void* weights, int n_tokens, int top,
-                              int n_experts, int inner, int shared, int columns, void* out, int dtype, hipStream_t stream) {
+                              int n_experts, int inner, int shared, int columns, void* out, int dtype,
+                              const void* shared_weight, hipStream_t stream) {
   const size_t total = (size_t)n_tokens * columns;
   if (total == 0) return 0;
   if (columns < n_experts * inner + shared) return -1;
   if (dtype == DT_BF16 && inner % 8 == 0 && shared % 8 == 0 && columns % 8 == 0 &&
       (((uintptr_t)gate_up | (uintptr_t)out) & 15) == 0) {
     expert_gate_vec_kernel<<<rt_blocks(total / 8), 256, 0, stream>>>((const bf16_t*)gate_up, (const int*)chosen,
-        (const float*)weights, top, n_experts, inner, shared, columns, (bf16_t*)out, total / 8);
+        (const float*)weights, top, n_experts, inner, shared, columns, (bf16_t*)out, total / 8, (const float*)shared_weight);
     return LAUNCH_STATUS();
   }
   if (dtype == DT_F32)
     expert_gate_kernel<float><<<rt_blocks(total), 256, 0, stream>>>((const float*)gate_up, (const int*)chosen,
-        (const float*)weights, top, n_experts, inner, shared, columns, (float*)out, total);
+        (const float*)weights, top, n_experts, inner, shared, columns, (float*)out, total, (const float*)shared_weight);
   else
     expert_gate_kernel<bf16_t><<<rt_blocks(total), 256, 0, stream>>>((const bf16_t*)gate_up, (const int*)chosen,
-        (const float*)weights, top, n_experts, inner, shared, columns, (bf16_t*)out, total);
+        (const float*)weights, top, n_experts, inner, shared, columns, (bf16_t*)out, total, (const float*)shared_weight);
   return LAUNCH_STATUS();
 }
 
@@ -339,7 +342,7 @@ extern "C" int ta_gelu_gate(const void* in, void* out, int n_tokens, int inner, 
 // the same values); `store` says whether this wave writes the token's results.
 __device__ __forceinline__ void rs_choose(float* choice, const float* score, float* worth, int lane, int n_experts,
                                           int n_groups, int keep, int top, bool store, int* __restrict__ chosen_row,
-                                          float* __restrict__ weights_row) {
+                                          float* __restrict__ weights_row, bool group_max = false) {
   if (n_groups > 0) {
     const int per = n_experts / n_groups;
     for (int g = lane; g < n_groups; g += WAVE) {
@@ -349,7 +352,7 @@ __device__ __forceinline__ void rs_choose(float* choice, const float* score, flo
         if (v > first) { second = first; first = v; }
         else if (v > second) second = v;
       }
-      worth[g] = per > 1 ? first + second : first;
+      worth[g] = (per > 1 && !group_max) ? first + second : first;
     }
     __syncthreads();
     for (int g = lane; g < n_groups; g += WAVE) {
@@ -411,6 +414,42 @@ route_sigmoid_kernel(const float* __restrict__ logits, const float* __restrict__
   }
   __syncthreads();
   rs_choose(choice, score, worth, lane, n_experts, n_groups, keep, top, live, chosen + (size_t)t * top, weights + (size_t)t * top);
+}
+
+// The same choice from scores of either kind.  logits: float rows of `stride` numbers, the experts' first.  softmax: the
+// scores are the softmax over all experts (else sigmoid); correction may be null; group_max: a group is worth its
+// largest choice score (else the sum of its two largest); gate (float [n_tokens] or null) gets sigmoid of the number
+// behind the experts' logits in the row.  A wave a token.
+__global__ void __launch_bounds__(256)
+route_scores_kernel(const float* __restrict__ logits, int stride, const float* __restrict__ correction, int n_tokens,
+                    int n_experts, int n_groups, int keep, int top, int softmax, int group_max, int* __restrict__ chosen,
+                    float* __restrict__ weights, float* __restrict__ gate) {
+  extern __shared__ float rs_scratch[];
+  const int lane = threadIdx.x & (WAVE - 1), wave = threadIdx.x / WAVE;
+  const int slot = blockIdx.x * (blockDim.x / WAVE) + wave;
+  const bool live = slot < n_tokens;                          // (a wave past the end works on the last token and stores nothing)
+  const int t = live ? slot : n_tokens - 1;
+  float* choice = rs_scratch + (size_t)wave * (2 * n_experts + n_groups);
+  float* score = choice + n_experts;
+  float* worth = score + n_experts;
+  const float* row = logits + (size_t)t * stride;
+  float top_logit = -INFINITY, total = 1.f;
+  if (softmax) {
+    for (int e = lane; e < n_experts; e += WAVE) top_logit = fmaxf(top_logit, row[e]);
+    top_logit = wave_max(top_logit);
+    total = 0.f;
+    for (int e = lane; e < n_experts; e += WAVE) total += expf(row[e] - top_logit);
+    total = wave_sum(total);
+  }
+  for (int e = lane; e < n_experts; e += WAVE) {
+    const float s = softmax ? expf(row[e] - top_logit) / total : 1.0f / (1.0f + expf(-row[e]));
+    score[e] = s;
+    choice[e] = correction ? s + correction[e] : s;
+  }
+  if (gate && live && lane == 0) gate[t] = 1.0f / (1.0f + expf(-row[n_experts]));
+  __syncthreads();
+  rs_choose(choice, score, worth, lane, n_experts, n_groups, keep, top, live, chosen + (size_t)t * top,
+            weights + (size_t)t * top, group_max != 0);
 }
 
 // The router's product and the choice in one kernel, a token a workgroup (few rows: a decode step): as route_rows_kernel
@@ -538,6 +577,19 @@ extern "C" int ta_route_sigmoid(const void* logits, const void* correction, int 
   const size_t lds = (size_t)4 * (2 * n_experts + n_groups) * sizeof(float);
   route_sigmoid_kernel<<<(n_tokens + 3) / 4, 256, lds, stream>>>((const float*)logits, (const float*)correction, n_tokens,
                                                                  n_experts, n_groups, keep, top, (int*)chosen, (float*)weights);
+  return LAUNCH_STATUS();
+}
+
+extern "C" int ta_route_scores(const void* logits, int stride, const void* correction, int n_tokens, int n_experts,
+                               int n_groups, int keep, int top, int softmax, int group_max, void* chosen, void* weights,
+                               void* gate, hipStream_t stream) {
+  if (n_tokens <= 0) return 0;
+  if (top <= 0 || top > n_experts || top > WAVE || n_experts > RS_MAX_EXPERTS || n_groups < 0) return -1;
+  if (stride < n_experts + (gate ? 1 : 0)) return -1;
+  if (n_groups > 0 && (n_experts % n_groups || keep <= 0 || keep > n_groups || keep * (n_experts / n_groups) < top)) return -1;
+  const size_t lds = (size_t)4 * (2 * n_experts + n_groups) * sizeof(float);
+  route_scores_kernel<<<(n_tokens + 3) / 4, 256, lds, stream>>>((const float*)logits, stride, (const float*)correction,
+      n_tokens, n_experts, n_groups, keep, top, softmax, group_max, (int*)chosen, (float*)weights, (float*)gate);
   return LAUNCH_STATUS();
 }
 

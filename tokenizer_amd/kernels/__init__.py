@@ -157,7 +157,8 @@ class Ops:
                      "ta_capped_gate", "ta_norm_add_rmsnorm", "ta_norm_rotate_store", "ta_differential_heads",
                      "ta_sigmoid_head_gate", "ta_route_top", "ta_expert_gate", "ta_side_gate", "ta_gelu_gate", "ta_norm_side_norm", "ta_route_rows", "ta_expert_slots", "ta_grouped_gemm_bf16", "ta_expert_combine",
                      "ta_add_pair_rmsnorm", "ta_latent_store", "ta_rotate_tails", "ta_head_linear", "ta_short_conv_silu",
-                     "ta_delta_scan", "ta_route_sigmoid", "ta_route_rows_sigmoid", "ta_expert_act", "ta_relu2"):
+                     "ta_delta_scan", "ta_route_sigmoid", "ta_route_rows_sigmoid", "ta_expert_act", "ta_relu2",
+                     "ta_add_terms_rmsnorm", "ta_scale_cap", "ta_route_scores", "ta_selective_scan"):
             getattr(self.lib, name).restype = ctypes.c_int
         self.lib.ta_grouped_gemm_bf16.argtypes = [ctypes.c_void_p, ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int,
                                                   ctypes.c_int, ctypes.c_void_p, ctypes.c_long, ctypes.c_int, ctypes.c_void_p,
@@ -364,13 +365,13 @@ class Ops:
     # ---------------------------------------------------- delta rule with a decay per key channel
     def short_conv_silu(self, rows: torch.Tensor, offsets, widths, taps: torch.Tensor, state: torch.Tensor, state_offset: int,
                         cu_q: torch.Tensor, first_position: torch.Tensor, state_slots: torch.Tensor,
-                        entry_of_token: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
-        """A short causal convolution over time, channel by channel, then silu.  The channels are up to three runs of
+                        entry_of_token: torch.Tensor, out: torch.Tensor, bias: torch.Tensor | None = None) -> torch.Tensor:
+        """A short causal convolution over time, channel by channel, (+ bias, float32 [channels],) then silu.  The channels are up to three runs of
         columns of `rows` (run i: widths[i] columns from offsets[i] on), side by side in `out` [T, channels]; taps float32
         [channels, n_taps], the last column the current token's.  Inputs before an entry's first row are its state row's
         [state_offset : + (n_taps - 1) channels] (oldest first; zeros if its first position is 0), which then takes the
         entry's last n_taps - 1 inputs."""
-        _dev(rows, taps, state, cu_q, first_position, state_slots, entry_of_token, out)
+        _dev(rows, taps, state, cu_q, first_position, state_slots, entry_of_token, out, bias)
         offsets, widths = [int(o) for o in offsets], [int(w) for w in widths]
         _need(len(offsets) == len(widths) and 1 <= len(widths) <= 3, "one to three runs of channels")
         while len(widths) < 3:
@@ -387,12 +388,114 @@ class Ops:
               "out is [T, channels]")
         n_entries = cu_q.numel() - 1
         _need(first_position.numel() == n_entries == state_slots.numel(), "one first position and slot per entry")
+        _need(bias is None or (bias.dtype == torch.float32 and bias.numel() == channels and bias.is_contiguous()),
+              "the bias is float32 [channels]")
         self._check(self.lib.ta_short_conv_silu(_ptr(rows), rows.shape[1], offsets[0], widths[0], offsets[1], widths[1],
                                                 offsets[2], widths[2], _ptr(taps), n_taps, _ptr(state),
                                                 ctypes.c_long(state.shape[1]), state_offset, _ptr(cu_q), _ptr(first_position),
                                                 _ptr(state_slots), _ptr(entry_of_token), _ptr(out), n_tokens, n_entries,
-                                                _code(rows.dtype), self._stream()), "short_conv_silu")
+                                                _code(rows.dtype), _ptr(bias), self._stream()), "short_conv_silu")
         return out
+
+    def selective_scan(self, x: torch.Tensor, pre: torch.Tensor, neg_rate: torch.Tensor, low: torch.Tensor, b_offset: int,
+                       c_offset: int, skip: torch.Tensor, rows: torch.Tensor, z_offset: int, state: torch.Tensor,
+                       cu_q: torch.Tensor, first_position: torch.Tensor, state_slots: torch.Tensor, out: torch.Tensor,
+                       channels: int, n: int) -> torch.Tensor:
+        """The selective scan over every entry's rows, from and into the entries' state rows (their first channels * n
+        numbers; zeros if the entry's first position is 0).  Per channel c and state j, with d = softplus(pre[t, c]):
+        S[c, j] <- exp(d neg_rate[c, j]) S[c, j] + d x[t, c] B[t, j]; y = sum_j S[c, j] C[t, j] + skip[c] x[t, c];
+        out[t, c] = y * silu(z[t, c]).  x [T, channels]; pre float32 [T, channels]; neg_rate float32 [channels, n]; B and C
+        are the columns b_offset.. and c_offset.. of `low`; z the columns z_offset.. of `rows`; out [T, channels]."""
+        _dev(x, pre, neg_rate, low, skip, rows, state, cu_q, first_position, state_slots, out)
+        n_tokens = x.shape[0]
+        _need(x.dim() == 2 and x.shape[1] >= channels and x.stride(1) == 1, "x is [T, >= channels]")
+        _need(pre.dtype == torch.float32 and tuple(pre.shape) == (n_tokens, channels) and pre.is_contiguous(),
+              "the step sizes' pre-activations are float32 [T, channels]")
+        _need(neg_rate.dtype == torch.float32 and tuple(neg_rate.shape) == (channels, n) and neg_rate.is_contiguous(),
+              "the rates are float32 [channels, n]")
+        _need(skip.dtype == torch.float32 and skip.numel() == channels, "the skip weights are float32 [channels]")
+        _need(low.dtype == x.dtype and low.shape[0] == n_tokens and low.stride(1) == 1
+              and 0 <= b_offset and b_offset + n <= low.shape[1] and 0 <= c_offset and c_offset + n <= low.shape[1],
+              "B and C do not fit the narrow rows")
+        _need(rows.dtype == x.dtype and rows.shape[0] == n_tokens and rows.stride(1) == 1 and 0 <= z_offset
+              and z_offset + channels <= rows.shape[1], "z does not fit the rows")
+        _need(tuple(out.shape) == (n_tokens, channels) and out.dtype == x.dtype and out.is_contiguous(), "out is [T, channels]")
+        _need(state.dtype == torch.float32 and state.dim() == 2 and state.shape[1] >= channels * n and state.is_contiguous(),
+              "state rows are too short")
+        _need(0 < n <= 256, "up to 256 numbers of state a channel")
+        n_entries = cu_q.numel() - 1
+        _need(first_position.numel() == n_entries == state_slots.numel(), "one first position and slot per entry")
+        self._check(self.lib.ta_selective_scan(_ptr(x), x.stride(0), _ptr(pre), _ptr(neg_rate), _ptr(low), low.stride(0),
+                                               int(b_offset), int(c_offset), _ptr(skip), _ptr(rows), rows.stride(0),
+                                               int(z_offset), _ptr(state), ctypes.c_long(state.shape[1]), _ptr(cu_q),
+                                               _ptr(first_position), _ptr(state_slots), _ptr(out), n_entries, channels, n,
+                                               _code(x.dtype), self._stream()), "selective_scan")
+        return out
+
+    def add_terms_rmsnorm(self, residual: torch.Tensor, terms, weight: torch.Tensor | None, eps: float, out: torch.Tensor,
+                          rows: torch.Tensor | None = None, store_residual: bool = True, weight2: torch.Tensor | None = None,
+                          eps2: float = 0.0, out2: torch.Tensor | None = None) -> torch.Tensor:
+        """x = residual[r] + sum_k factor_k * scale_k * rows_k[r] in float32 (`terms`: up to four of (rows [T, H] in out's
+        dtype, factor, scale float32 [H] or None)); optionally residual[r] = x; out[i] = rmsnorm(x) * weight (weight None:
+        out[i] = x; out may be a view whose rows lie further apart than H); with out2, a second normalised copy under
+        weight2 and eps2.  rows int32 [R] picks the rows (None: all)."""
+        terms = tuple(terms)
+        n_tokens, hidden = residual.shape
+        n_rows = n_tokens if rows is None else rows.numel()
+        _dev(residual, weight, rows, weight2, out2)
+        _need(out.is_cuda, "kernel operands must live on the GPU")       # (its rows may lie apart: a half of wider rows)
+        _need(len(terms) <= 4, "up to four terms")
+        _need(residual.dtype == torch.float32 and residual.is_contiguous(), "the residual stream is float32")
+        for term, _, scale in terms:
+            _dev(term, scale)
+            _need(tuple(term.shape) == (n_tokens, hidden) and term.dtype == out.dtype and term.is_contiguous(),
+                  "a term is [T, H] in the output's dtype")
+            _need(scale is None or (scale.dtype == torch.float32 and scale.numel() == hidden and scale.is_contiguous()),
+                  "a term's scale is float32 [H]")
+        for w in (weight, weight2):
+            _need(w is None or (w.dtype == torch.float32 and w.numel() == hidden), "norm weight must be float32 [H]")
+        _need(tuple(out.shape) == (n_rows, hidden) and out.stride(1) == 1 and out.stride(0) >= hidden, "norm output has the wrong shape")
+        _need(out2 is None or (weight2 is not None and tuple(out2.shape) == (n_rows, hidden) and out2.dtype == out.dtype
+                               and out2.is_contiguous()), "the second output is [R, H] with a weight of its own")
+        _need(rows is None or (rows.dtype == torch.int32 and not store_residual), "rows int32, and a subset stores nothing back")
+        _need(hidden <= 8192, "rows of up to 8192 elements")
+        filled = list(terms) + [(None, 0.0, None)] * (4 - len(terms))
+        self._check(self.lib.ta_add_terms_rmsnorm(
+            _ptr(residual), len(terms), *[_ptr(t[0]) for t in filled], *[_ptr(t[2]) for t in filled],
+            *[ctypes.c_float(float(t[1])) for t in filled], _ptr(weight), ctypes.c_float(eps), _ptr(out), out.stride(0),
+            _ptr(weight2), ctypes.c_float(eps2), _ptr(out2), _ptr(rows), n_rows, hidden, int(bool(store_residual)),
+            _code(out.dtype), self._stream()), "add_terms_rmsnorm")
+        return out
+
+    def scale_cap(self, x: torch.Tensor, scale: float, cap: float) -> torch.Tensor:
+        """x <- cap * tanh(scale * x / cap) in place (cap 0: scale * x); x float32."""
+        _dev(x)
+        _need(x.dtype == torch.float32 and x.is_contiguous(), "float32 rows")
+        self._check(self.lib.ta_scale_cap(_ptr(x), ctypes.c_size_t(x.numel()), ctypes.c_float(scale), ctypes.c_float(cap),
+                                          self._stream()), "scale_cap")
+        return x
+
+    def route_scores(self, logits: torch.Tensor, correction: torch.Tensor | None, n_experts: int, n_groups: int,
+                     keep_groups: int, chosen: torch.Tensor, weights: torch.Tensor, softmax: bool = False,
+                     group_max: bool = False, gate: torch.Tensor | None = None) -> None:
+        """As `route_sigmoid`, from scores of either kind: float32 `logits` [T, >= n_experts] (the experts' first);
+        `softmax`: s = softmax over all experts (else sigmoid); `correction` may be None; `group_max`: a group is worth
+        its largest choice score (else its two largest); `gate` (float32 [T]) gets sigmoid of the number behind the
+        experts' logits in a row."""
+        _dev(logits, correction, chosen, weights, gate)
+        n_tokens, top = logits.shape[0], chosen.shape[1]
+        _need(logits.dtype == torch.float32 and logits.is_contiguous() and logits.shape[1] >= n_experts + (gate is not None),
+              "router logits are float32 [T, >= experts]")
+        _need(correction is None or (correction.dtype == torch.float32 and correction.numel() == n_experts), "the correction is float32")
+        _need(chosen.dtype == torch.int32 and weights.dtype == torch.float32
+              and tuple(chosen.shape) == (n_tokens, top) == tuple(weights.shape), "chosen int32 and weights float32 [T, top]")
+        _need(gate is None or (gate.dtype == torch.float32 and gate.numel() == n_tokens), "the gate is float32 [T]")
+        _need(0 < top <= min(n_experts, 64) and n_experts <= 1024, "between one and 64 of up to 1024 experts a token")
+        _need(n_groups == 0 or (n_experts % n_groups == 0 and 0 < keep_groups <= n_groups
+                                and keep_groups * (n_experts // n_groups) >= top), "the groups do not fit")
+        self._check(self.lib.ta_route_scores(_ptr(logits), logits.shape[1], _ptr(correction), n_tokens, n_experts, int(n_groups),
+                                             int(keep_groups), top, int(bool(softmax)), int(bool(group_max)), _ptr(chosen),
+                                             _ptr(weights), _ptr(gate), self._stream()), "route_scores")
 
     def delta_scan(self, fresh: torch.Tensor, decay: torch.Tensor, neg_rate: torch.Tensor, rows: torch.Tensor, beta_offset: int,
                    state: torch.Tensor, cu_q: torch.Tensor, first_position: torch.Tensor, state_slots: torch.Tensor,
@@ -695,8 +798,8 @@ class Ops:
         return out
 
     def expert_combine(self, rows: torch.Tensor, slot_of: torch.Tensor, weights: torch.Tensor, shared: torch.Tensor | None,
-                       out: torch.Tensor) -> torch.Tensor:
-        """out[t] = shared[t] (if given) + sum over the token's picks of weights[t, k] * rows[slot_of[t top + k]]; rows
+                       out: torch.Tensor, shared_weight: torch.Tensor | None = None) -> torch.Tensor:
+        """out[t] = shared[t] (if given; times shared_weight[t], float32 [T], if that is given) + sum over the token's picks of weights[t, k] * rows[slot_of[t top + k]]; rows
         float32 [slots, H], weights float32 [T, top], shared and out [T, H] of one dtype."""
         _dev(rows, slot_of, weights, shared, out)
         n_tokens, top = weights.shape
@@ -705,16 +808,21 @@ class Ops:
               and weights.is_contiguous(), "slot_of int32 [T top], weights float32 [T, top]")
         _need(out.is_contiguous() and out.shape[0] == n_tokens and (shared is None or (shared.shape == out.shape
               and shared.dtype == out.dtype and shared.is_contiguous())), "shared and out are [T, H]")
+        _dev(shared_weight)
+        _need(shared_weight is None or (shared_weight.dtype == torch.float32 and shared_weight.numel() == n_tokens),
+              "the shared expert's weights are float32 [T]")
         self._check(self.lib.ta_expert_combine(_ptr(rows), _ptr(slot_of), _ptr(weights), n_tokens, top, _ptr(shared), _ptr(out),
-                                               out.shape[1], _code(out.dtype), self._stream()), "expert_combine")
+                                               out.shape[1], _code(out.dtype), _ptr(shared_weight), self._stream()), "expert_combine")
         return out
 
     def expert_gate(self, gate_up: torch.Tensor, chosen: torch.Tensor, weights: torch.Tensor, n_experts: int, inner: int,
-                    shared: int, out: torch.Tensor) -> torch.Tensor:
+                    shared: int, out: torch.Tensor, shared_weight: torch.Tensor | None = None) -> torch.Tensor:
         """gate_up [T, n_experts 2 inner + 2 shared] (every expert's gate rows, then its up rows; the shared expert
         last) -> out [T, >= n_experts inner + shared]: weight * silu(gate) * up in the columns of the experts a token
-        chose, silu(gate) * up in the shared expert's, zero everywhere else."""
-        _dev(gate_up, chosen, weights, out)
+        chose, silu(gate) * up in the shared expert's (times shared_weight[t], float32 [T], if given), zero everywhere else."""
+        _dev(gate_up, chosen, weights, out, shared_weight)
+        _need(shared_weight is None or (shared_weight.dtype == torch.float32 and shared_weight.numel() == gate_up.shape[0]),
+              "the shared expert's weights are float32 [T]")
         n_tokens = gate_up.shape[0]
         _need(gate_up.is_contiguous() and gate_up.shape[1] == n_experts * 2 * inner + 2 * shared, "gate_up width")
         _need(out.is_contiguous() and out.shape[0] == n_tokens and out.shape[1] >= n_experts * inner + shared
@@ -722,8 +830,8 @@ class Ops:
         _need(chosen.dtype == torch.int32 and weights.dtype == torch.float32 and chosen.shape == weights.shape
               and chosen.shape[0] == n_tokens and chosen.is_contiguous() and weights.is_contiguous(), "chosen and weights [T, top]")
         self._check(self.lib.ta_expert_gate(_ptr(gate_up), _ptr(chosen), _ptr(weights), n_tokens, chosen.shape[1], n_experts,
-                                            inner, shared, out.shape[1], _ptr(out), _code(out.dtype), self._stream()),
-                    "expert_gate")
+                                            inner, shared, out.shape[1], _ptr(out), _code(out.dtype), _ptr(shared_weight),
+                                            self._stream()), "expert_gate")
         return out
 
     def side_gate(self, gate: torch.Tensor, table: torch.Tensor, token_ids: torch.Tensor, offset: int, dim: int,
@@ -814,8 +922,10 @@ class Ops:
                         window: int | None, scale: float, max_position: int | None = None,
                         batch=None, value_dim: int | None = None, chunk: int | None = None,
                         slopes: torch.Tensor | None = None, sinks: torch.Tensor | None = None,
-                        keep_first: int = 0, value_heads: int | None = None) -> torch.Tensor:
+                        keep_first: int = 0, value_heads: int | None = None, softcap: float | None = None) -> torch.Tensor:
         """Causal attention of every token over the pages of its request.
+
+        `softcap` c: a score (scaled, with its distance term) becomes c tanh(score / c) before the softmax.
 
         `keep_first` n (with a window): keys at positions below n stay visible behind the window.  `value_heads`
         (a divisor of n_kv): the value pages hold so many heads, and key head g reads value head
@@ -859,7 +969,7 @@ class Ops:
         # heads go to the generic kernel.
         plain = plain and keep_first == 0 and value_heads == n_kv
         if (value_dim == head_dim and qkv.dtype == torch.bfloat16 and head_dim in self.DECODE_HEAD_DIMS and page_size % 16 == 0
-                and qkv.shape[1] % 8 == 0 and self.use_fast_attention
+                and qkv.shape[1] % 8 == 0 and self.use_fast_attention and not softcap
                 and (keep_first == 0 or (chunk is None and slopes is None))):
             args = (qkv, out, k_pages, v_pages, positions, entry_of_token, block_table, n_q, n_kv, head_dim,
                     page_size, window, scale, max_position)
@@ -897,7 +1007,7 @@ class Ops:
             _ptr(entry_of_token), _ptr(block_table), block_table.shape[1], n_tokens, n_q, n_kv, head_dim,
             page_size, -1 if window is None else int(window), ctypes.c_float(scale), _code(qkv.dtype),
             value_dim, 0 if chunk is None else int(chunk), _ptr(slopes), _ptr(sinks), keep_first, value_heads,
-            self._stream()), "paged_attention")
+            ctypes.c_float(softcap or 0.0), self._stream()), "paged_attention")
         return out
 
     DECODE_HEAD_DIMS = (16, 32, 48, 64, 80, 96, 112, 128, 160, 192, 224, 256)
