@@ -64,15 +64,17 @@ def capped_sink_attention(h: torch.Tensor, m: dict, w: dict) -> torch.Tensor:
     q = (h @ w["q"].T + w["q.b"]).reshape(T, H, d)
     k = (h @ w["k"].T + w["k.b"]).reshape(T, G, d)
     v = (h @ w["v"].T + w["v.b"]).reshape(T, G, dv)
-    rot = m["rot"]
-    q = rotate_leading(q, positions, int(rot["dims"]), float(rot["base"]))
-    k = rotate_leading(k, positions, int(rot["dims"]), float(rot["base"]))
+    rot = m.get("rot")
+    if rot:
+        q = rotate_leading(q, positions, int(rot["dims"]), float(rot["base"]))
+        k = rotate_leading(k, positions, int(rot["dims"]), float(rot["base"]))
     out = torch.zeros((T, H, dv), dtype=h.dtype)
     for head in range(H):
         g = head // (H // G)
         for t in range(T):
             s = (k[:t + 1, g] @ q[t, head]) * float(m["scale"])
-            s = cap(s, float(m["softcap"]))
+            if m.get("softcap") is not None:
+                s = cap(s, float(m["softcap"]))
             sink = w["sink"][head]
             top = torch.maximum(s.max(), sink)
             e = torch.exp(s - top)
@@ -176,7 +178,7 @@ def run_order(cfg: dict) -> list[tuple[int, bool]]:
 def forward(cfg: dict, tensors: dict, ids: list[int], layers_out: list | None = None) -> torch.Tensor:
     """Logits [T, vocab] of the whole sequence `ids`; `layers_out` collects the stream behind every layer run."""
     eps = float(cfg["norm"]["eps"])
-    x0 = tensors["embed"][torch.tensor(ids)] * float(cfg["embedding"]["scale"])
+    x0 = tensors["embed"][torch.tensor(ids)] * float((cfg.get("embedding") or {}).get("scale", 1.0))
     x = x0
     for index, pass_starts in run_order(cfg):
         if pass_starts:
@@ -195,8 +197,8 @@ def forward(cfg: dict, tensors: dict, ids: list[int], layers_out: list | None = 
         x = x + y
         if layers_out is not None:
             layers_out.append(x.clone())
-    logits = rms_norm(x, tensors["final.norm"], eps) @ tensors["head"].T * float(cfg["logit_scale"])
-    return cap(logits, float(cfg["logit_softcap"]))
+    logits = rms_norm(x, tensors["final.norm"], eps) @ tensors["head"].T * float(cfg.get("logit_scale") or 1.0)
+    return cap(logits, float(cfg["logit_softcap"])) if cfg.get("logit_softcap") else logits
 
 
 def greedy_generate(cfg: dict, tensors: dict, prompt, n_new: int) -> list[int]:
