@@ -77,7 +77,7 @@ def zomavik_spec(cfg: ZomavikConfig) -> ModelSpec:
         else:
             schedule.append(ScheduleEntry(index))
             seen.add(index)
-    options = {"logit_scale": cfg.logit_scale, "logit_cap": cfg.logit_softcap}
+    options = {"head_scale": cfg.logit_scale, "head_cap": cfg.logit_softcap}
     if starts:
         options["pass_input"] = {"tensor": "loop.in", "before": tuple(starts)}
     return ModelSpec(

@@ -211,12 +211,12 @@ class DecoderModel:
         # Options of the frame.  `pass_input` {"tensor": name, "before": schedule indices}: in front of those scheduled
         # layers the stream x becomes W [x; x0] with W [hidden, 2 hidden] and x0 the embedding's output (a run of
         # layers that is gone through several times takes the token in again at the start of every pass).
-        # `logit_scale` s and `logit_cap` c: the logits are c tanh(s z / c).
+        # `head_scale` s and `head_cap` c: the logits are c tanh(s z / c).
         pass_input = spec.options.get("pass_input") or {}
         self.pass_before = frozenset(int(index) for index in pass_input.get("before", ()))
         self.pass_weight = tensors[pass_input["tensor"]] if self.pass_before else None
-        self.logit_scale = float(spec.options.get("logit_scale") or 1.0)
-        self.logit_cap = float(spec.options.get("logit_cap") or 0.0)
+        self.logit_scale = float(spec.options.get("head_scale") or 1.0)
+        self.logit_cap = float(spec.options.get("head_cap") or 0.0)
         self.final_norm = NORMS.get(spec.final_norm.kind)(spec.final_norm, _strip(spec.final_norm_prefix, tensors), runtime)
         self.head = self.embedding if spec.tied_head else tensors[spec.head_name]
         parts = [self.final_norm] + [p for b in self.blocks if hasattr(b, "mixer")
