@@ -18,7 +18,7 @@ share a prefix of 1,024 ids, with the prefix cache) and prints one JSON line for
 
 times the prompt attention kernel alone on a portion of TOKENS tokens after C cached ones.
 
-    python bench.py --design napadra|dolidra|bokulorn [--size 0.5b|1.5b|7b] [--layers N] [--batch B] [--steps K]
+    python bench.py --design napadra|dolidra|bokulorn|zomavik [--size 0.5b|1.5b|7b] [--layers N] [--batch B] [--steps K]
 
 times a prefill of 2,048 tokens and decoding at batch B of a Napadra model whose layers have the sizes of the
 Qwen2.5 model named (width, heads, feed-forward and vocabulary; its layers alternate attention, attention on the
@@ -64,10 +64,23 @@ def weight_bytes_per_step(model) -> int:
     seen, total = set(), 0
     decoder = model.decoder
     tensors = [decoder.head]
+
+    def held(part):
+        """The tensors a part holds, and those of the parts it is made of (two mixers side by side)."""
+        for value in vars(part).values():
+            if isinstance(value, torch.Tensor):
+                tensors.append(value)
+            elif isinstance(value, (list, tuple)):
+                for item in value:
+                    if hasattr(item, "forward") and hasattr(item, "__dict__"):
+                        held(item)
+
+    if getattr(decoder, "pass_weight", None) is not None:
+        tensors.append(decoder.pass_weight)
     for block in decoder.blocks:
         for part in (block.mixer_norm, block.mixer, block.feed_forward_norm, block.feed_forward):
             if part is not None:
-                tensors.extend(v for v in vars(part).values() if isinstance(v, torch.Tensor))
+                held(part)
     tensors.extend(v for v in vars(decoder.final_norm).values() if isinstance(v, torch.Tensor))
     for tensor in tensors:
         if tensor.data_ptr() not in seen:
@@ -327,18 +340,45 @@ def bokulorn_config(sizes: dict, layers: int, experts: int = 8, top: int = 2) ->
             "embedding": {"scale": 1.0}, "layers": out}
 
 
+def zomavik_config(sizes: dict, layers: int, experts: int = 8, top: int = 2) -> dict:
+    """A Zomavik configuration with the layer sizes of a Qwen2 one: `layers` layer runs, of which two layers run twice.
+    Every layer's mixer is an attention with Qwen2's heads (values as wide as keys, the whole head rotated, capped scores,
+    a sink) beside a selective scan over as many channels as the width, sixteen numbers of state a channel; the first
+    layer's feed-forward is dense, the others route `top` of `experts` gated experts of half the dense inner width (as
+    many multiply-adds a token as the gated dense one) in four groups of which two are kept, with a gated shared expert
+    of a quarter."""
+    width, heads, kv_heads = sizes["hidden_size"], sizes["num_attention_heads"], sizes["num_key_value_heads"]
+    d, inner = width // heads, sizes["intermediate_size"]
+    mixer = {"left": {"heads": heads, "kv_heads": kv_heads, "dim": d, "vdim": d, "scale": d ** -0.5, "softcap": 30.0,
+                      "rot": {"dims": d, "base": float(sizes.get("rope_theta", 1e6))}},
+             "right": {"inner": width, "state": 16, "dt_rank": max(8, width // 16 // 8 * 8), "conv": 4},
+             "left_scale": 0.6, "right_scale": 0.5}
+    moe = {"kind": "moe", "expert": {"ff": inner // 2 // 8 * 8}, "shared": {"ff": inner // 4 // 8 * 8},
+           "router": {"experts": experts, "top": top, "groups": {"count": 4, "keep": 2}}}
+    out = [{"type": "parallel", "mixer": mixer, "mlp": {"kind": "dense", "ff": inner} if index == 0 else moe}
+           for index in range(layers)]
+    loop = {"start": 1, "stop": 3, "times": 2} if layers >= 3 else {"start": 0, "stop": layers, "times": 2}
+    return {"architecture": "Zomavik", "vocab": sizes["vocab_size"], "width": width, "norm": {"eps": 1e-6},
+            "embedding": {"scale": 1.0}, "logit_scale": 1.0, "logit_softcap": 30.0, "loop": loop, "layers": out}
+
+
 def run_design(args, sizes: dict) -> dict:
-    """Prefill and decode throughput of the named design beside its closest neighbour (Qwen2; for Bokulorn, Dolidra, whose
+    """Prefill and decode throughput of the named design beside its closest neighbour (Qwen2; for Zomavik, Bokulorn, whose layers also set a recurrence with
+    its state in the request's slot beside attention and routed experts; for Bokulorn, Dolidra, whose
     layers also mix attention with routed experts) at equal layer sizes and number of layer runs."""
     import torch
-    from tokenizer_amd.config import BokulornConfig, DolidraConfig, NapadraConfig, Qwen2Config
+    from tokenizer_amd.config import BokulornConfig, DolidraConfig, NapadraConfig, Qwen2Config, ZomavikConfig
     from tokenizer_amd.engine import random_model
     layers = args.layers or 8
     steps = min(args.steps, 256)
-    beside = "dolidra" if args.design == "bokulorn" else "qwen2"
+    beside = {"bokulorn": "dolidra", "zomavik": "bokulorn"}.get(args.design, "qwen2")
     record = {"design": args.design, "beside": beside, "size": args.size, "layers": layers, "dtype": args.dtype,
               "prompt_len": PROMPT_LEN, "batch": args.batch, "decode_steps": steps, "data": "synthetic (random weights)"}
-    if args.design == "bokulorn":
+    if args.design == "zomavik":
+        # (Two of Zomavik's layers run twice: `layers` counts the runs, so that both models run as many layers a token.)
+        configs = {"zomavik": lambda: ZomavikConfig.from_dict(zomavik_config(sizes, max(2, layers - 2))),
+                   "bokulorn": lambda: BokulornConfig.from_dict(bokulorn_config(sizes, layers))}
+    elif args.design == "bokulorn":
         configs = {"bokulorn": lambda: BokulornConfig.from_dict(bokulorn_config(sizes, layers)),
                    "dolidra": lambda: DolidraConfig.from_dict(dolidra_config(sizes, max(2, layers - 2)))}
     elif args.design == "dolidra":
@@ -459,9 +499,9 @@ def main() -> int:
     parser.add_argument("--layers", type=int, default=None)
     parser.add_argument("--size", default="0.5b", choices=["0.5b", "1.5b", "7b"],
                         help="layer sizes of the decode benchmark (the default is the one the record is for)")
-    parser.add_argument("--design", default=None, choices=["napadra", "dolidra", "bokulorn"],
+    parser.add_argument("--design", default=None, choices=["napadra", "dolidra", "bokulorn", "zomavik"],
                         help="time this design beside its closest neighbour at equal layer sizes (prefill and decode)")
-    parser.add_argument("--only", default=None, choices=["napadra", "dolidra", "bokulorn", "qwen2"], help="with --design: one of the two models")
+    parser.add_argument("--only", default=None, choices=["napadra", "dolidra", "bokulorn", "zomavik", "qwen2"], help="with --design: one of the two models")
     parser.add_argument("--peaks", action="store_true", help="measure what the device reaches in HBM reads and bf16 products")
     parser.add_argument("--workload", default=None, choices=["mixed-1.5b", "mixed-0.5b", "prefix-7b"],
                         help="run a serving workload through the scheduler instead of the decode benchmark")

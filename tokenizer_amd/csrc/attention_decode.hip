@@ -33,7 +33,8 @@ __device__ __forceinline__ bf16x8 zero8() {
 // key head g reads value head g / (n_kv / n_v).
 // EXTRA: chunk > 0: only the keys of the token's own run of `chunk` positions (runs counted from position 0) are seen;
 // slopes (float [n_q] or null): head h's score loses slopes[h] per position between token and key; sinks (float [n_q] or
-// null): exp(sinks[h]) joins the softmax's denominator (it rides in the first split's partial sums).
+// null): exp(sinks[h]) joins the softmax's denominator (it rides in the first split's partial sums); softcap > 0: a
+// score s (scaled, with its distance term) becomes softcap * tanh(s / softcap).
 template <int D, int DEC_WAVES, bool AHEAD, bool EXTRA>
 __global__ void __launch_bounds__(DEC_WAVES * WAVE)
 decode_attention_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __restrict__ out,
@@ -43,7 +44,7 @@ decode_attention_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __re
                         int table_stride, float* __restrict__ part_o, float* __restrict__ part_ml,
                         int n_q, int n_kv, int page_size, int window, float scale, int split_keys, int splits,
                         int chunk, const float* __restrict__ slopes, const float* __restrict__ sinks,
-                        int keep_first, int kept_splits, int n_v) {
+                        int keep_first, int kept_splits, int n_v, float softcap) {
   constexpr int KS = (D + 31) / 32;   // 32-wide steps over the head size for Q K^T
   constexpr int DB = D / 16;          // 16-row blocks of O^T
   HELD(q, q_stride, out, k_pages, vt_pages, rows, positions, entry_of_token, block_table, table_stride, part_o, part_ml,
@@ -190,6 +191,7 @@ decode_attention_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __re
         const int key = kb + 8 * g + 4 * t + r;
         float score = st[r] * scale;
         if (EXTRA) score = fmaf(-slope, (float)(pos - key), score);
+        if (EXTRA && softcap > 0.f) score = softcap * (1.f - 2.f / (1.f + __expf(2.f * score / softcap)));
         s[t][r] = (blk.active && key >= lo && key <= last) ? score : -INFINITY;
       }
     }
@@ -373,7 +375,7 @@ static int launch_decode(const void* q, int q_stride, void* out, const void* k_p
                          const void* block_table, int table_stride, void* part_o, void* part_ml, int n_items,
                          int n_q, int n_kv, int page_size, int window, float scale, int split_keys, int splits,
                          int chunk, const void* slopes, const void* sinks, int keep_first, int kept_splits, int n_v,
-                         hipStream_t stream) {
+                         float softcap, hipStream_t stream) {
   const int group = n_q / n_kv;
   dim3 grid(splits, n_kv * ((group + 15) / 16), n_items);
   constexpr int NW = D > 128 ? 2 : 4;   // keeps the merge buffer within 64 KB of LDS
@@ -381,8 +383,8 @@ static int launch_decode(const void* q, int q_stride, void* out, const void* k_p
       (const bf16_t*)q, q_stride, (bf16_t*)out, (const bf16_t*)k_pages, (const bf16_t*)vt_pages, (const int*)rows, \
       (const int*)positions, (const int*)entry_of_token, (const int*)block_table, table_stride, (float*)part_o, \
       (float*)part_ml, n_q, n_kv, page_size, window, scale, split_keys, splits, chunk, (const float*)slopes, \
-      (const float*)sinks, keep_first, kept_splits, n_v)
-  if (chunk > 0 || slopes || sinks || kept_splits > 0 || (n_v > 0 && n_v < n_kv)) { if (split_keys <= 32 * NW * 8) GO(true, true); else GO(false, true); }
+      (const float*)sinks, keep_first, kept_splits, n_v, softcap)
+  if (chunk > 0 || slopes || sinks || kept_splits > 0 || softcap > 0.f || (n_v > 0 && n_v < n_kv)) { if (split_keys <= 32 * NW * 8) GO(true, true); else GO(false, true); }
   else if (split_keys <= 32 * NW * 8) GO(true, false); else GO(false, false);      // up to eight blocks a wave
 #undef GO
   int status = LAUNCH_STATUS();
@@ -414,7 +416,7 @@ extern "C" int ta_decode_attention_bf16(const void* q, int q_stride, void* out, 
                                         void* part_o, void* part_ml, int n_items, int n_q, int n_kv, int d,
                                         int page_size, int window, float scale, int split_keys, int splits,
                                         int chunk, const void* slopes, const void* sinks, int keep_first,
-                                        int kept_splits, int n_v, hipStream_t stream) {
+                                        int kept_splits, int n_v, float softcap, hipStream_t stream) {
   if (n_items <= 0) return 0;
   if (n_kv <= 0 || n_q % n_kv || page_size % 16 || split_keys % 32 || splits < 1) return -1;
   if (n_v <= 0) n_v = n_kv;
@@ -423,7 +425,7 @@ extern "C" int ta_decode_attention_bf16(const void* q, int q_stride, void* out, 
     return -1;
 #define CASE(DD) case DD: return launch_decode<DD>(q, q_stride, out, k_pages, vt_pages, rows, positions, entry_of_token, \
     block_table, table_stride, part_o, part_ml, n_items, n_q, n_kv, page_size, window, scale, split_keys, splits, chunk, \
-    slopes, sinks, keep_first, kept_splits, n_v, stream);
+    slopes, sinks, keep_first, kept_splits, n_v, softcap, stream);
   switch (d) {
     CASE(16) CASE(32) CASE(48) CASE(64) CASE(80) CASE(96) CASE(112) CASE(128) CASE(160) CASE(192) CASE(224) CASE(256)
     default: return -2;

@@ -23,13 +23,13 @@ __device__ __forceinline__ bf16x8 pf_zero8() {
 // the wave.  FULL: every key of the block is visible to every token of the tile, so nothing is masked.
 // Scores stay unscaled; `c` = scale * log2(e) enters in exp2(s*c - m*c).
 // EXTRA: head h's score (still unscaled) loses `slope[h]` (the head's slope over the scale) per position between the
-// token and the key.
+// token and the key; then, with cap > 0 (the scores' cap over the scale), the score s becomes cap * tanh(s / cap).
 template <int D, int HG, bool FULL, bool EXTRA>
 __device__ __forceinline__ void prefill_block(
     const bf16_t* __restrict__ k_pages, const bf16_t* __restrict__ vt_pages, const int* __restrict__ table,
     int kb, int kvh, int n_kv, int page_size, int col, int g, int heads_here, int my_pos, int my_lo, int lo, int hi,
     float c, const bf16x8 (&qf)[HG][(D + 31) / 32], floatx4 (&acc)[HG][D / 16], float (&m)[HG], float (&l)[HG],
-    const float (&slope)[HG], int keep_first = 0, int vh = -1, int n_vh = 0) {
+    const float (&slope)[HG], int keep_first = 0, int vh = -1, int n_vh = 0, float cap = 0.f) {
   // EXTRA: keep_first > 0: keys below it stay visible (and their pages readable) behind the window; vh >= 0: the
   // value pages hold n_vh heads and this key head reads value head vh.
   if (!EXTRA || vh < 0) { vh = kvh; n_vh = n_kv; }
@@ -117,6 +117,7 @@ __device__ __forceinline__ void prefill_block(
         const int key = kb + 32 * (t >> 1) + 8 * g + 4 * (t & 1) + r;     // (keys outside lo..hi lie outside my_lo..my_pos)
         float score = st[r];
         if (EXTRA) score = fmaf(-slope[h], (float)(my_pos - key), score);
+        if (EXTRA && cap > 0.f) score = cap * (1.f - 2.f / (1.f + __expf(2.f * score / cap)));
         if (FULL) {
           s[t * 4 + r] = score;
         } else {
@@ -168,7 +169,7 @@ prefill_attention_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __r
                          const int* __restrict__ first_position, const int* __restrict__ block_table,
                          int table_stride, int n_q, int n_kv, int page_size, int window, float scale_log2,
                          int chunk, const float* __restrict__ slopes, const float* __restrict__ sinks, float inv_scale,
-                         int keep_first, int n_v) {
+                         int keep_first, int n_v, float softcap) {
   constexpr int KS = (D + 31) / 32;
   constexpr int DB = D / 16;
   HELD(q, q_stride, out, k_pages, vt_pages, tiles, n_tiles, cu_q, first_position, block_table, table_stride, n_q, n_kv,
@@ -255,18 +256,18 @@ prefill_attention_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __r
     const int kept_end = min(kept, (lo / 64) * 64);
     for (int k0 = 64 * wave; k0 < kept_end; k0 += 64 * NWV)
       prefill_block<D, HG, false, EXTRA>(k_pages, vt_pages, table, k0, kvh, n_kv, page_size, col, g, heads_here, my_pos,
-                                  my_lo, lo, hi, scale_log2, qf, acc, m, l, slope, kept, vh, n_vh);
+                                  my_lo, lo, hi, scale_log2, qf, acc, m, l, slope, kept, vh, n_vh, softcap * inv_scale);
   }
   int kb = (lo / 64) * 64 + 64 * wave;
   for (; kb <= hi && kb < lo_all; kb += 64 * NWV)
     prefill_block<D, HG, false, EXTRA>(k_pages, vt_pages, table, kb, kvh, n_kv, page_size, col, g, heads_here, my_pos,
-                                my_lo, lo, hi, scale_log2, qf, acc, m, l, slope, kept, vh, n_vh);
+                                my_lo, lo, hi, scale_log2, qf, acc, m, l, slope, kept, vh, n_vh, softcap * inv_scale);
   for (; kb + 63 <= p0; kb += 64 * NWV)
     prefill_block<D, HG, true, EXTRA>(k_pages, vt_pages, table, kb, kvh, n_kv, page_size, col, g, heads_here, my_pos,
-                               my_lo, lo, hi, scale_log2, qf, acc, m, l, slope, kept, vh, n_vh);
+                               my_lo, lo, hi, scale_log2, qf, acc, m, l, slope, kept, vh, n_vh, softcap * inv_scale);
   for (; kb <= hi; kb += 64 * NWV)
     prefill_block<D, HG, false, EXTRA>(k_pages, vt_pages, table, kb, kvh, n_kv, page_size, col, g, heads_here, my_pos,
-                                my_lo, lo, hi, scale_log2, qf, acc, m, l, slope, kept, vh, n_vh);
+                                my_lo, lo, hi, scale_log2, qf, acc, m, l, slope, kept, vh, n_vh, softcap * inv_scale);
   if (NWV > 1) {
     // Waves 1.. hand their state to wave 0: maximum, sum and the output accumulators of each head.
     if (wave > 0) {
@@ -346,6 +347,7 @@ struct PrefillExtras {       // what the plain form does not have: see ta_prefil
   const float* sinks;
   int keep_first;            // with a window: keys below this stay visible behind it
   int n_v;                   // value heads in the value pages (0 or n_kv: one a key head)
+  float softcap;             // > 0: a scaled score s becomes softcap * tanh(s / softcap)
 };
 
 template <int D, int HG, int NWV>
@@ -359,8 +361,8 @@ static int launch_prefill_waves(const void* q, int q_stride, void* out, const vo
 #define GO(EE) prefill_attention_kernel<D, HG, NWV, EE><<<(unsigned)workgroups, NWV * WAVE, 0, stream>>>( \
       (const bf16_t*)q, q_stride, (bf16_t*)out, (const bf16_t*)k_pages, (const bf16_t*)vt_pages, (const int*)tiles, \
       n_tiles, (const int*)cu_q, (const int*)first_position, (const int*)block_table, table_stride, n_q, n_kv, page_size, \
-      window, scale * 1.4426950408889634f, extra.chunk, extra.slopes, extra.sinks, 1.0f / scale, extra.keep_first, extra.n_v)
-  if (extra.chunk > 0 || extra.slopes || extra.sinks || extra.keep_first > 0 || (extra.n_v > 0 && extra.n_v < n_kv)) GO(true);
+      window, scale * 1.4426950408889634f, extra.chunk, extra.slopes, extra.sinks, 1.0f / scale, extra.keep_first, extra.n_v, extra.softcap)
+  if (extra.chunk > 0 || extra.slopes || extra.sinks || extra.keep_first > 0 || extra.softcap > 0.f || (extra.n_v > 0 && extra.n_v < n_kv)) GO(true);
   else GO(false);
 #undef GO
   return LAUNCH_STATUS();
@@ -454,13 +456,13 @@ extern "C" int ta_prefill_attention_bf16(const void* q, int q_stride, void* out,
                                          int n_q, int n_kv, int d, int page_size, int window, float scale,
                                          int shared_shape, int max_keys, int waves, int shared,
                                          void* part_o, void* part_ml, int chunk, const void* slopes, const void* sinks,
-                                         int keep_first, int n_v, hipStream_t stream) {
+                                         int keep_first, int n_v, float softcap, hipStream_t stream) {
   if (n_tiles <= 0) return 0;
   if (n_kv <= 0 || n_q % n_kv || page_size % 16 || scale == 0.f) return -1;
   if (n_v <= 0) n_v = n_kv;
   if (n_kv % n_v || keep_first < 0 || (keep_first > 0 && (window < 0 || chunk > 0 || slopes))) return -1;
-  const PrefillExtras extra = {chunk, (const float*)slopes, (const float*)sinks, keep_first, n_v};
-  const bool plain = chunk <= 0 && !slopes && !sinks && keep_first == 0 && n_v == n_kv;
+  const PrefillExtras extra = {chunk, (const float*)slopes, (const float*)sinks, keep_first, n_v, softcap};
+  const bool plain = chunk <= 0 && !slopes && !sinks && keep_first == 0 && n_v == n_kv && !(softcap > 0.f);
   const int shape = plain ? shared_shape_for(n_tiles, n_q, n_kv, d, window, shared_shape, max_keys, waves, shared) : 0;
   if (shape) {
     const int parts = (part_o && part_ml)

@@ -969,12 +969,13 @@ class Ops:
         # heads go to the generic kernel.
         plain = plain and keep_first == 0 and value_heads == n_kv
         if (value_dim == head_dim and qkv.dtype == torch.bfloat16 and head_dim in self.DECODE_HEAD_DIMS and page_size % 16 == 0
-                and qkv.shape[1] % 8 == 0 and self.use_fast_attention and not softcap
+                and qkv.shape[1] % 8 == 0 and self.use_fast_attention
                 and (keep_first == 0 or (chunk is None and slopes is None))):
             args = (qkv, out, k_pages, v_pages, positions, entry_of_token, block_table, n_q, n_kv, head_dim,
                     page_size, window, scale, max_position)
+            plain = plain and not softcap
             extras = {} if plain else dict(chunk=chunk, slopes=slopes, sinks=sinks, keep_first=keep_first,
-                                           value_heads=value_heads)
+                                           value_heads=value_heads, softcap=softcap)
             if batch is None:
                 return self._decode_attention(*args, **extras)
             if batch.q_tiles.numel() == 0:
@@ -998,7 +999,7 @@ class Ops:
                 n_tiles, _ptr(batch.cu_q), _ptr(batch.first_position), _ptr(block_table),
                 block_table.shape[1], n_q, n_kv, head_dim, page_size, choice[0], ctypes.c_float(scale), *choice[1:],
                 _ptr(part_o), _ptr(part_ml), 0 if chunk is None else int(chunk), _ptr(slopes), _ptr(sinks),
-                keep_first, value_heads, self._stream()), "prefill_attention")
+                keep_first, value_heads, ctypes.c_float(softcap or 0.0), self._stream()), "prefill_attention")
             if batch.decode_rows.numel():
                 self._decode_attention(*args, rows=batch.decode_rows, **extras)
             return out
@@ -1025,7 +1026,8 @@ class Ops:
 
     def _decode_attention(self, qkv, out, k_pages, v_pages, positions, entry_of_token, block_table,
                           n_q, n_kv, head_dim, page_size, window, scale, max_position, rows=None,
-                          identity_entries=False, chunk=None, slopes=None, sinks=None, keep_first=0, value_heads=None):
+                          identity_entries=False, chunk=None, slopes=None, sinks=None, keep_first=0, value_heads=None,
+                          softcap=None):
         """Matrix-core attention of single tokens with the key range split over workgroups (kept first keys behind a
         window are further splits of their own)."""
         n_items = qkv.shape[0] if rows is None else rows.numel()
@@ -1055,7 +1057,7 @@ class Ops:
             n_q, n_kv, head_dim, page_size, -1 if window is None else int(window), ctypes.c_float(scale),
             split_keys, splits, 0 if chunk is None else int(chunk), _ptr(slopes), _ptr(sinks),
             int(keep_first) if kept_splits else 0, kept_splits, n_kv if value_heads is None else int(value_heads),
-            self._stream()), "decode_attention")
+            ctypes.c_float(softcap or 0.0), self._stream()), "decode_attention")
         return out
 
     # --------------------------------------------------------------------- linear
