@@ -302,6 +302,29 @@ def test_selective_scan_alone(backend, cut, width, inner, state, rank, taps):
 
 
 @pytest.mark.parametrize("backend", BACKENDS)
+@pytest.mark.parametrize("width,inner,state,rank,taps", [(64, 128, 16, 8, 4), (40, 36, 7, 5, 2), (32, 24, 40, 6, 3)])
+def test_long_portions_run_in_chunks_side_by_side(backend, width, inner, state, rank, taps):
+    """Portions of hundreds of tokens are cut into chunks whose states are carried from one to the next: a prompt of 300
+    (no multiple of a chunk), a single token, a portion of 267 that starts from the state those left, then single tokens;
+    a second request's portion of 150 rides in the first step, so the two entries' chunks lie side by side."""
+    ops, device, dtype = ops_for(backend)
+    gen = torch.Generator().manual_seed(inner + state)
+    n = 600
+    w = scan_tensors(gen, width, inner, state, rank, taps, dtype, size=2.0, rate=-1.0, step=-2.0)
+    h = rounded(torch.randn(n, width, generator=gen, dtype=torch.float64), dtype)
+    other = rounded(torch.randn(150, width, generator=gen, dtype=torch.float64), dtype)
+    m = {"inner": inner, "state": state, "dt_rank": rank, "conv": taps}
+    want, want_other = plain.selective_scan(h, m, w), plain.selective_scan(other, m, w)
+    runner = PartRunner("selective_scan", scan_spec(width, inner, state, rank, taps), w, backend, num_pages=60)
+    first = runner.step([("other", other), ("main", h[:300])])
+    rest = runner.run(h[300:], [1, 267] + [1] * 32, rider=other[:5])
+    got = torch.cat([first[1], rest])
+    bound = tolerance(dtype, 3e-5, 6e-2)
+    assert float((first[0] - want_other).abs().max()) <= bound * max(1.0, float(want_other.abs().max()))
+    assert float((got - want).abs().max()) <= bound * max(1.0, float(want.abs().max()))
+
+
+@pytest.mark.parametrize("backend", BACKENDS)
 @pytest.mark.parametrize("cut", list(CUTS))
 def test_a_write_that_is_read_two_hundred_tokens_later(backend, cut):
     """Decays of nearly one (rates and step sizes far down) keep what a token wrote: the first tokens' inputs are made

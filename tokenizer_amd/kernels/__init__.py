@@ -425,12 +425,25 @@ class Ops:
         _need(0 < n <= 256, "up to 256 numbers of state a channel")
         n_entries = cu_q.numel() - 1
         _need(first_position.numel() == n_entries == state_slots.numel(), "one first position and slot per entry")
+        # Steps with long portions cut them into chunks that run side by side (the choice depends on the step's counts
+        # alone, so a captured step makes it as an eager one does).
+        chunk = self.SCAN_CHUNK if n_tokens >= self.SCAN_CHUNKED_FROM else 0
+        max_chunks, chunk_state, chunk_sum = 0, None, None
+        if chunk:
+            max_chunks = -(-n_tokens // chunk)
+            slots = n_tokens // chunk + n_entries + 1
+            chunk_state = torch.empty((slots, channels * n), dtype=torch.float32, device=x.device)
+            chunk_sum = torch.empty((slots, channels), dtype=torch.float32, device=x.device)
         self._check(self.lib.ta_selective_scan(_ptr(x), x.stride(0), _ptr(pre), _ptr(neg_rate), _ptr(low), low.stride(0),
                                                int(b_offset), int(c_offset), _ptr(skip), _ptr(rows), rows.stride(0),
                                                int(z_offset), _ptr(state), ctypes.c_long(state.shape[1]), _ptr(cu_q),
                                                _ptr(first_position), _ptr(state_slots), _ptr(out), n_entries, channels, n,
-                                               _code(x.dtype), self._stream()), "selective_scan")
+                                               _code(x.dtype), chunk, max_chunks, _ptr(chunk_state), _ptr(chunk_sum),
+                                               self._stream()), "selective_scan")
         return out
+
+    SCAN_CHUNK = 64             # tokens a chunk of the selective scan's chunked form
+    SCAN_CHUNKED_FROM = 192     # tokens in a step from which the chunked form runs
 
     def add_terms_rmsnorm(self, residual: torch.Tensor, terms, weight: torch.Tensor | None, eps: float, out: torch.Tensor,
                           rows: torch.Tensor | None = None, store_residual: bool = True, weight2: torch.Tensor | None = None,
