@@ -153,7 +153,7 @@ def test_greedy_generation_through_the_entry_point_and_the_scheduler(folders, ba
 @pytest.mark.gpu
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 @pytest.mark.parametrize("cut", ["whole", "tail", "portions", "mixed"])
-@pytest.mark.parametrize("name", ["C", "A"])
+@pytest.mark.parametrize("name", ["C", "A", "E"])
 def test_hundreds_of_tokens(folders, oracle, dtype, cut, name):
     """Prompts long enough for the prompt kernels' tiles, the sorted routed layers and a long walk of the scan."""
     reqs = requests_for(name, (300, 17, 411, 130))

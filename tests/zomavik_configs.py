@@ -61,6 +61,8 @@ _B = [_mixer(_left(3, 3, 10, 14, 6, 300.0, 0.35, 5.0), _right(36, 7, 5, 2), 1.2,
 _C = [_mixer(_left(4, 1, 64, 64, 32, 500000.0, 0.125, 30.0), _right(128, 16, 8, 4), 0.6, 0.5),
       _mixer(_left(8, 2, 32, 32, 32, 10000.0, 0.18, 12.0), _right(256, 24, 16, 3), 0.9, 0.2)]
 _D = [_mixer(_left(1, 1, 24, 40, 2, 100.0, 0.2, 3.0), _right(16, 1, 1, 1), 1.0, 1.0)]
+_E = [_mixer(_left(5, 5, 12, 6, 10, 2000.0, 0.29, 7.0), _right(30, 11, 3, 3), 0.8, 0.6),
+      _mixer(_left(2, 1, 18, 22, 18, 50.0, 0.24, 40.0), _right(54, 20, 7, 4), 0.45, 0.9)]
 
 ZOMAVIK = {
     # name: (config.json keys, weight seed)
@@ -81,6 +83,10 @@ ZOMAVIK = {
         _layer(_C[0], _dense(96))], scale=11.3, loop=(0, 1, 3), logit_scale=2.0, logit_softcap=25.0), 21),
     # One tap (no convolution state), one head, a rotation of one pair, one number of state, a step-size rank of one,
     # weights of 1 on both sides, an embedding as it is, a run that is gone through once, scaled logits without a cap.
+    # A width that is no multiple of four under a repeated run (the pass's input is a row of twice that width), an odd
+    # vocabulary, the whole model gone through twice, seven experts without groups, twenty numbers of state.
+    "E": (_model(131, 50, 1e-5, [_layer(_E[0], _moe(7, 3, 18, shared=10)), _layer(_E[1], _dense(34)), _layer(_E[0])],
+                 scale=6.0, loop=(0, 3, 2), logit_scale=1.5, logit_softcap=12.0), 55),
     "D": (_model(120, 40, 1e-6, [_layer(_D[0], _moe(3, 1, 16, 3, 1)), _layer(_D[0], _dense(24))], loop=(0, 2, 1),
                  logit_scale=0.7), 34),
 }

@@ -459,7 +459,7 @@ template <typename T>
 __global__ void __launch_bounds__(256)
 route_rows_sigmoid_kernel(const T* __restrict__ x, int lda, const T* __restrict__ router, const float* __restrict__ correction,
                           int hidden, int n_experts, int n_groups, int keep, int top, int* __restrict__ chosen,
-                          float* __restrict__ weights) {
+                          float* __restrict__ weights, int softmax = 0, int group_max = 0, float* __restrict__ gate = nullptr) {
   constexpr int N = RtVec<T>::N;
   extern __shared__ float rs_scratch[];
   float* choice = rs_scratch;
@@ -477,7 +477,8 @@ route_rows_sigmoid_kernel(const T* __restrict__ x, int lda, const T* __restrict_
 #pragma unroll
       for (int k = 0; k < N; ++k) xv[p][k] = 0.f;
   }
-  for (int e = wave; e < n_experts; e += 256 / WAVE) {
+  // (With a gate, the router has one row more: the gate's, behind the experts'.)
+  for (int e = wave; e < n_experts + (gate ? 1 : 0); e += 256 / WAVE) {
     const T* w = router + (size_t)e * hidden;
     float sum = 0.f;
 #pragma unroll
@@ -492,14 +493,32 @@ route_rows_sigmoid_kernel(const T* __restrict__ x, int lda, const T* __restrict_
     }
     sum = wave_sum(sum);
     if (lane == 0) {
-      const float s = 1.0f / (1.0f + expf(-sum));
-      score[e] = s;
-      choice[e] = s + correction[e];
+      if (e == n_experts) {
+        gate[t] = 1.0f / (1.0f + expf(-sum));
+      } else if (softmax) {
+        score[e] = sum;                                      // the logit, until all of them are there
+      } else {
+        const float s = 1.0f / (1.0f + expf(-sum));
+        score[e] = s;
+        choice[e] = correction ? s + correction[e] : s;
+      }
     }
   }
   __syncthreads();
+  if (softmax) {                                             // every thread sums the few logits up for itself
+    float top_logit = -INFINITY, total = 0.f;
+    for (int e = 0; e < n_experts; ++e) top_logit = fmaxf(top_logit, score[e]);
+    for (int e = 0; e < n_experts; ++e) total += expf(score[e] - top_logit);
+    __syncthreads();
+    for (int e = threadIdx.x; e < n_experts; e += 256) {
+      const float s = expf(score[e] - top_logit) / total;
+      score[e] = s;
+      choice[e] = correction ? s + correction[e] : s;
+    }
+    __syncthreads();
+  }
   rs_choose(choice, score, worth, lane, n_experts, n_groups, keep, top, wave == 0, chosen + (size_t)t * top,
-            weights + (size_t)t * top);
+            weights + (size_t)t * top, group_max != 0);
 }
 
 // up: [n_tokens, n_experts * inner]; out: [n_tokens, columns], columns >= n_experts * inner:
@@ -590,6 +609,29 @@ extern "C" int ta_route_scores(const void* logits, int stride, const void* corre
   const size_t lds = (size_t)4 * (2 * n_experts + n_groups) * sizeof(float);
   route_scores_kernel<<<(n_tokens + 3) / 4, 256, lds, stream>>>((const float*)logits, stride, (const float*)correction,
       n_tokens, n_experts, n_groups, keep, top, softmax, group_max, (int*)chosen, (float*)weights, (float*)gate);
+  return LAUNCH_STATUS();
+}
+
+// The same for scores of either kind (see route_scores_kernel): router [n_experts (+ 1 with a gate), hidden].
+extern "C" int ta_route_rows_scores(const void* x, int lda, const void* router, const void* correction, int n_tokens,
+                                    int hidden, int n_experts, int n_groups, int keep, int top, int softmax, int group_max,
+                                    void* chosen, void* weights, void* gate, int dtype, hipStream_t stream) {
+  if (n_tokens <= 0) return 0;
+  if (top <= 0 || top > n_experts || top > WAVE || n_groups < 0) return -1;
+  if (n_groups > 0 && (n_experts % n_groups || keep <= 0 || keep > n_groups || keep * (n_experts / n_groups) < top)) return -1;
+  const int piece = dtype == DT_F32 ? 4 : 8;
+  if (n_experts > RT_MAX_EXPERTS || hidden % piece || lda % piece || hidden > WAVE * RT_ROW_PIECES * piece ||
+      (((uintptr_t)x | (uintptr_t)router) & 15))
+    return -2;
+  const size_t lds = (size_t)(2 * n_experts + n_groups) * sizeof(float);
+  if (dtype == DT_F32)
+    route_rows_sigmoid_kernel<float><<<n_tokens, 256, lds, stream>>>((const float*)x, lda, (const float*)router,
+        (const float*)correction, hidden, n_experts, n_groups, keep, top, (int*)chosen, (float*)weights, softmax, group_max,
+        (float*)gate);
+  else
+    route_rows_sigmoid_kernel<bf16_t><<<n_tokens, 256, lds, stream>>>((const bf16_t*)x, lda, (const bf16_t*)router,
+        (const float*)correction, hidden, n_experts, n_groups, keep, top, (int*)chosen, (float*)weights, softmax, group_max,
+        (float*)gate);
   return LAUNCH_STATUS();
 }
 

@@ -107,10 +107,19 @@ selective_scan_kernel(const T* __restrict__ x, int x_stride, const float* __rest
     }
   };
 
+  // Where finished rows wait for the threads that write them out: sixteen tokens by sixteen channels.
+  __shared__ float s_out[SS_STAGE][SS_CH];
+  auto write_out = [&](int t0) {                             // thread (token, channel) of the stage that lies in s_out
+    const int t = t0 + f_token;
+    if (t < hi && f_channel < channels) st(out + (size_t)t * channels + f_channel, s_out[f_token][threadIdx.x % SS_CH]);
+  };
+
   fetch(lo);
   for (int t0 = lo; t0 < hi; t0 += SS_STAGE) {
-    __syncthreads();                                         // the stage before has been read
-    s_dt[f_token][threadIdx.x % SS_CH] = ss_softplus(r_pre);
+    __syncthreads();                                         // the stage before has been read, its rows lie in s_out
+    if (MODE != SS_LOCAL && t0 > lo) write_out(t0 - SS_STAGE);
+    // (A token past the portion's end gets a step size of zero and zeros all round: it leaves the state as it is.)
+    s_dt[f_token][threadIdx.x % SS_CH] = t0 + f_token < hi ? ss_softplus(r_pre) : 0.f;
     s_x[f_token][threadIdx.x % SS_CH] = r_x;
     s_z[f_token][threadIdx.x % SS_CH] = r_z;
 #pragma unroll
@@ -120,9 +129,9 @@ selective_scan_kernel(const T* __restrict__ x, int x_stride, const float* __rest
     }
     __syncthreads();
     if (t0 + SS_STAGE < hi) fetch(t0 + SS_STAGE);            // under way while this stage is worked on
-    const int count = min(SS_STAGE, hi - t0);
-#pragma unroll 4
-    for (int tt = 0; tt < count; ++tt) {
+    float ys[SS_STAGE];
+#pragma unroll
+    for (int tt = 0; tt < SS_STAGE; ++tt) {
       const float step = s_dt[tt][mine], xv = s_x[tt][mine];
       const float in = step * xv;
       float y = 0.f;
@@ -132,16 +141,44 @@ selective_scan_kernel(const T* __restrict__ x, int x_stride, const float* __rest
         S[r] = fmaf(__expf(step * a[r]), S[r], in * s_b[tt][j]);
         y = fmaf(S[r], s_c[tt][j], y);
       }
-      if (MODE == SS_LOCAL) {
-        sum += step;
-      } else {
-        y = ss_row_sum16(y);
-        if (part == 0 && live) {
-          const float gate = s_z[tt][mine];
-          st(out + (size_t)(t0 + tt) * channels + c, fmaf(skip, xv, y) * (gate / (1.0f + __expf(-gate))));
-        }
-      }
+      ys[tt] = y;
+      if (MODE == SS_LOCAL) sum += step;
     }
+    if (MODE != SS_LOCAL) {
+      // Sixteen lanes hold sixteen tokens' parts each; four exchanges (with the lane 1, 2, 4 and 8 away, halving what is
+      // held each time) leave lane i with token i's whole sum, which it gates and puts down.
+#define SS_XOR1(v) __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0xB1, 0xF, 0xF, false))
+#define SS_XOR2(v) __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x4E, 0xF, 0xF, false))
+#define SS_XOR8(v) __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x128, 0xF, 0xF, false))
+      const bool b0 = part & 1, b1 = part & 2, b2 = part & 4, b3 = part & 8;
+      float v8[8], v4[4], v2[2];
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        const float keep = b0 ? ys[2 * i + 1] : ys[2 * i], send = b0 ? ys[2 * i] : ys[2 * i + 1];
+        v8[i] = keep + SS_XOR1(send);
+      }
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const float keep = b1 ? v8[2 * i + 1] : v8[2 * i], send = b1 ? v8[2 * i] : v8[2 * i + 1];
+        v4[i] = keep + SS_XOR2(send);
+      }
+#pragma unroll
+      for (int i = 0; i < 2; ++i) {
+        const float keep = b2 ? v4[2 * i + 1] : v4[2 * i], send = b2 ? v4[2 * i] : v4[2 * i + 1];
+        v2[i] = keep + __shfl_xor(send, 4, WAVE);
+      }
+      const float keep = b3 ? v2[1] : v2[0], send = b3 ? v2[0] : v2[1];
+      const float y = keep + SS_XOR8(send);
+#undef SS_XOR1
+#undef SS_XOR2
+#undef SS_XOR8
+      const float gate = s_z[part][mine];
+      s_out[part][mine] = fmaf(skip, s_x[part][mine], y) * (gate / (1.0f + __expf(-gate)));
+    }
+  }
+  if (MODE != SS_LOCAL) {
+    __syncthreads();
+    write_out(lo + (hi - lo - 1) / SS_STAGE * SS_STAGE);
   }
   if (!live) return;
   if (MODE == SS_LOCAL) {

@@ -158,7 +158,7 @@ class Ops:
                      "ta_sigmoid_head_gate", "ta_route_top", "ta_expert_gate", "ta_side_gate", "ta_gelu_gate", "ta_norm_side_norm", "ta_route_rows", "ta_expert_slots", "ta_grouped_gemm_bf16", "ta_expert_combine",
                      "ta_add_pair_rmsnorm", "ta_latent_store", "ta_rotate_tails", "ta_head_linear", "ta_short_conv_silu",
                      "ta_delta_scan", "ta_route_sigmoid", "ta_route_rows_sigmoid", "ta_expert_act", "ta_relu2",
-                     "ta_add_terms_rmsnorm", "ta_scale_cap", "ta_route_scores", "ta_selective_scan"):
+                     "ta_add_terms_rmsnorm", "ta_scale_cap", "ta_route_scores", "ta_selective_scan", "ta_route_rows_scores"):
             getattr(self.lib, name).restype = ctypes.c_int
         self.lib.ta_grouped_gemm_bf16.argtypes = [ctypes.c_void_p, ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int,
                                                   ctypes.c_int, ctypes.c_void_p, ctypes.c_long, ctypes.c_int, ctypes.c_void_p,
@@ -739,6 +739,35 @@ class Ops:
         if status == -2:
             return False
         self._check(status, "route_rows")
+        return True
+
+    def route_rows_scores(self, x: torch.Tensor, router: torch.Tensor, correction: torch.Tensor | None, n_experts: int,
+                          n_groups: int, keep_groups: int, chosen: torch.Tensor, weights: torch.Tensor, softmax: bool = False,
+                          group_max: bool = False, gate: torch.Tensor | None = None) -> bool:
+        """`route_scores` of the float32 logits x @ router.T without leaving them in memory (router [n_experts, H], or with
+        a gate [n_experts + 1, H], the gate's row last): product and choice in one kernel, a token a workgroup (for the few
+        rows of a decode step).  Returns False for sizes the kernel does not take: the caller then forms the logits with
+        `linear` and calls `route_scores`."""
+        _dev(x, router, correction, chosen, weights, gate)
+        n_tokens, hidden = x.shape
+        top = chosen.shape[1]
+        _need(x.dtype == router.dtype and x.stride(1) == 1 and router.is_contiguous() and router.shape[1] == hidden
+              and router.shape[0] == n_experts + (gate is not None), "router [E (+ 1), H]")
+        _need(correction is None or (correction.dtype == torch.float32 and correction.numel() == n_experts), "the correction is float32 [E]")
+        _need(chosen.dtype == torch.int32 and weights.dtype == torch.float32 and chosen.is_contiguous() and weights.is_contiguous()
+              and tuple(chosen.shape) == (n_tokens, top) == tuple(weights.shape), "chosen int32 and weights float32 [T, top]")
+        _need(gate is None or (gate.dtype == torch.float32 and gate.numel() == n_tokens), "the gate is float32 [T]")
+        _need(0 < top <= min(n_experts, 64), "between one and 64 experts a token, no more than there are")
+        _need(n_groups >= 0 and (n_groups == 0 or (n_experts % n_groups == 0 and 0 < keep_groups <= n_groups
+                                                   and keep_groups * (n_experts // n_groups) >= top)),
+              "the kept groups must hold the experts a token uses")
+        status = self.lib.ta_route_rows_scores(_ptr(x), x.stride(0) if n_tokens > 1 else hidden, _ptr(router), _ptr(correction),
+                                               n_tokens, hidden, n_experts, int(n_groups), int(keep_groups), top,
+                                               int(bool(softmax)), int(bool(group_max)), _ptr(chosen), _ptr(weights),
+                                               _ptr(gate), _code(x.dtype), self._stream())
+        if status == -2:
+            return False
+        self._check(status, "route_rows_scores")
         return True
 
     def route_rows_sigmoid(self, x: torch.Tensor, router: torch.Tensor, correction: torch.Tensor, n_groups: int,

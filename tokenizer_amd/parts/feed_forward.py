@@ -229,9 +229,13 @@ class RoutedExperts(FeedForward):
         elif self.scored:
             if self.shared_gate:
                 shared_weight = torch.empty((x.shape[0],), dtype=torch.float32, device=x.device)
-            ops.route_scores(ops.linear(x, self.w_router, out_dtype=torch.float32), self.correction, self.n_experts,
-                             self.n_groups, self.keep_groups, chosen, weights, softmax=not self.sigmoid,
-                             group_max=self.spec.group_worth == "max", gate=shared_weight)
+            kind = dict(softmax=not self.sigmoid, group_max=self.spec.group_worth == "max", gate=shared_weight)
+            fused = getattr(ops, "route_rows_scores", None)    # few rows: the router's product and the choice in one kernel
+            if (fused is None or x.shape[0] > ops.ROUTE_ROWS_FUSED
+                    or not fused(x, self.w_router, self.correction, self.n_experts, self.n_groups, self.keep_groups, chosen,
+                                 weights, **kind)):
+                ops.route_scores(ops.linear(x, self.w_router, out_dtype=torch.float32), self.correction, self.n_experts,
+                                 self.n_groups, self.keep_groups, chosen, weights, **kind)
         else:
             fused = getattr(ops, "route_rows", None)      # the router's product and the choice in one kernel, where there is one
             if fused is None or not fused(x, self.w_router, chosen, weights):
