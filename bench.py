@@ -349,10 +349,10 @@ def zomavik_config(sizes: dict, layers: int, experts: int = 8, top: int = 2) -> 
     of a quarter."""
     width, heads, kv_heads = sizes["hidden_size"], sizes["num_attention_heads"], sizes["num_key_value_heads"]
     d, inner = width // heads, sizes["intermediate_size"]
-    mixer = {"left": {"heads": heads, "kv_heads": kv_heads, "dim": d, "vdim": d, "scale": d ** -0.5, "softcap": 30.0,
+    mixer = {"left": {"heads": heads, "kv_heads": kv_heads, "dim": d, "vdim": d, "scale": d ** -0.5, "softcap": 50.0,
                       "rot": {"dims": d, "base": float(sizes.get("rope_theta", 1e6))}},
              "right": {"inner": width, "state": 16, "dt_rank": max(8, width // 16 // 8 * 8), "conv": 4},
-             "left_scale": 0.6, "right_scale": 0.5}
+             "left_scale": 0.7, "right_scale": 0.4}
     moe = {"kind": "moe", "expert": {"ff": inner // 2 // 8 * 8}, "shared": {"ff": inner // 4 // 8 * 8},
            "router": {"experts": experts, "top": top, "groups": {"count": 4, "keep": 2}}}
     out = [{"type": "parallel", "mixer": mixer, "mlp": {"kind": "dense", "ff": inner} if index == 0 else moe}

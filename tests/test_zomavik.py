@@ -275,7 +275,7 @@ def scan_tensors(gen, width, inner, state, rank, taps, dtype, size=1.0, rate=0.0
     return {name: (t.float().double() if t.dim() == 1 or name == "conv" else rounded(t, dtype)) for name, t in w.items()}
 
 
-SCAN_SIZES = [(48, 48, 5, 3, 4), (40, 36, 7, 5, 2), (32, 16, 1, 1, 1), (64, 128, 16, 8, 4), (64, 100, 24, 12, 3),
+SCAN_SIZES = [(48, 48, 5, 3, 4), (40, 36, 7, 5, 2), (32, 16, 1, 1, 1), (64, 128, 16, 8, 4), (64, 100, 20, 10, 3),
               (32, 24, 40, 6, 6), (32, 8, 130, 2, 2)]
 
 
@@ -476,7 +476,7 @@ def run_feed_forward(kind, spec, tensors, backend, x):
 
 
 @pytest.mark.parametrize("backend", BACKENDS)
-@pytest.mark.parametrize("experts,top,count,keep", [(12, 4, 2, 1), (6, 2, 3, 2), (5, 1, 5, 5), (8, 3, None, None), (64, 6, 8, 3),
+@pytest.mark.parametrize("experts,top,count,keep", [(12, 3, 2, 1), (6, 2, 3, 2), (5, 1, 5, 5), (8, 3, None, None), (64, 6, 8, 3),
                                                      (4, 4, 1, 1), (9, 2, 9, 3)])
 def test_the_router_against_a_choice_written_out_here(backend, experts, top, count, keep):
     """Softmax over all experts, a group worth its best expert, the best groups kept, the best experts inside them,
@@ -567,7 +567,7 @@ def test_weighted_terms_join_the_stream_under_one_or_two_norms(backend, hidden, 
     for k in range(n_terms):
         part = torch.randn(rows, hidden, generator=gen).to(dtype)
         scale = None if k == 1 else (1 + 0.3 * torch.randn(hidden, generator=gen))
-        factor = [0.6, 0.5, 1.0, -1.5][k]
+        factor = [0.7, 0.4, 1.0, -1.5][k]
         total += factor * part.double() * (1.0 if scale is None else scale.double())
         terms.append((part.to(device), factor, None if scale is None else scale.to(device)))
     w1, w2 = (1 + 0.3 * torch.randn(hidden, generator=gen)), (1 + 0.3 * torch.randn(hidden, generator=gen))
@@ -598,6 +598,6 @@ def test_weighted_terms_join_the_stream_under_one_or_two_norms(backend, hidden, 
 def test_scaled_and_capped_logits(backend):
     ops, device, dtype = ops_for(backend)
     z = (torch.randn(5, 333, generator=torch.Generator().manual_seed(1)) * 40).to(device)
-    capped = ops.scale_cap(z.clone(), 0.25, 15.0).double().cpu()
-    assert torch.allclose(capped, 15.0 * torch.tanh(z.double().cpu() * 0.25 / 15.0), atol=1e-5)
+    capped = ops.scale_cap(z.clone(), 0.3, 12.0).double().cpu()
+    assert torch.allclose(capped, 12.0 * torch.tanh(z.double().cpu() * 0.3 / 12.0), atol=1e-5)
     assert torch.allclose(ops.scale_cap(z.clone(), 0.7, 0.0).double().cpu(), z.double().cpu() * 0.7, atol=1e-5)

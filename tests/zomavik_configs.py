@@ -58,7 +58,7 @@ _A = [_mixer(_left(4, 2, 16, 24, 8, 10000.0, 0.3, 20.0), _right(48, 5, 3, 4), 0.
       _mixer(_left(2, 1, 32, 16, 32, 500.0, 0.2, 8.0), _right(40, 9, 6, 3), 0.3, 1.1)]
 _B = [_mixer(_left(3, 3, 10, 14, 6, 300.0, 0.35, 5.0), _right(36, 7, 5, 2), 1.2, 0.8),
       _mixer(_left(6, 2, 6, 10, 0, 100.0, 0.4, None), _right(20, 3, 2, 5), 0.5, 0.5)]
-_C = [_mixer(_left(4, 1, 64, 64, 32, 500000.0, 0.125, 30.0), _right(128, 16, 8, 4), 0.6, 0.5),
+_C = [_mixer(_left(4, 1, 64, 64, 32, 500000.0, 0.125, 28.0), _right(128, 16, 8, 4), 0.65, 0.45),
       _mixer(_left(8, 2, 32, 32, 32, 10000.0, 0.18, 12.0), _right(256, 24, 16, 3), 0.9, 0.2)]
 _D = [_mixer(_left(1, 1, 24, 40, 2, 100.0, 0.2, 3.0), _right(16, 1, 1, 1), 1.0, 1.0)]
 _E = [_mixer(_left(5, 5, 12, 6, 10, 2000.0, 0.29, 7.0), _right(30, 11, 3, 3), 0.8, 0.6),
@@ -135,10 +135,10 @@ def random_config(seed: int) -> dict:
         kv_heads = rng.choice([1, 1, 2, 3])
         left = _left(kv_heads * rng.choice([1, 2, 4]), kv_heads, dim, vdim, rng.choice([0, 2, dim // 2 // 2 * 2, dim]),
                      rng.choice([100.0, 10000.0, 500000.0]), rng.choice([dim ** -0.5, 0.2, 0.35]),
-                     rng.choice([None, 4.0, 15.0, 50.0]))
+                     rng.choice([None, 4.0, 18.0, 50.0]))
         right = _right(rng.choice([16, 24, 40, 64, 100]), rng.choice([1, 4, 8, 11, 16, 24, 40]), rng.choice([1, 3, 8, 12]),
                        rng.choice([1, 2, 3, 4, 6]))
-        mixer = _mixer(left, right, rng.choice([0.5, 0.6, 1.0]), rng.choice([0.4, 0.5, 1.3]))
+        mixer = _mixer(left, right, rng.choice([0.55, 0.7, 1.0]), rng.choice([0.4, 0.45, 1.3]))
         kind = rng.random()
         if kind < 0.2:
             mlp = None
@@ -157,5 +157,5 @@ def random_config(seed: int) -> dict:
         start = rng.randrange(len(layers))
         loop = (start, rng.randint(start + 1, len(layers)), rng.randint(1, 3))
     return _model(rng.choice([61, 128, 200, 333]), width, rng.choice([1e-6, 1e-5]), layers,
-                  scale=rng.choice([None, 5.0, width ** 0.5]), loop=loop, logit_scale=rng.choice([None, 0.25, 1.5]),
-                  logit_softcap=rng.choice([None, 10.0, 30.0]))
+                  scale=rng.choice([None, 5.0, width ** 0.5]), loop=loop, logit_scale=rng.choice([None, 0.3, 1.5]),
+                  logit_softcap=rng.choice([None, 10.0, 35.0]))
