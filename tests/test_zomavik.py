@@ -391,7 +391,8 @@ def part_names(w):
 ATTENTION_SIZES = [(48, 4, 2, 16, 24, 8, 10000.0, 0.3, 20.0), (40, 3, 3, 10, 14, 6, 300.0, 0.35, 2.0),
                    (32, 1, 1, 24, 40, 2, 100.0, 0.2, 3.0), (64, 4, 1, 64, 64, 32, 500000.0, 0.125, 30.0),
                    (64, 8, 2, 32, 32, 32, 10000.0, 0.18, 4.0), (48, 6, 2, 6, 10, 0, 100.0, 0.4, None),
-                   (64, 6, 1, 48, 16, 48, 10000.0, 0.144, 50.0)]
+                   (64, 6, 1, 48, 16, 48, 10000.0, 0.144, 50.0), (64, 2, 1, 128, 128, 64, 10000.0, 0.09, 9.0),
+                   (48, 6, 2, 96, 96, 96, 1000.0, 0.1, 6.0), (40, 3, 1, 80, 80, 10, 200.0, 0.11, None)]
 
 
 @pytest.mark.parametrize("backend", BACKENDS)
